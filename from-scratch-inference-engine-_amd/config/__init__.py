@@ -2,7 +2,8 @@
 
 from .base import ConfigError, ModelConfig, read_config_json
 from .botulorn import BotulornConfig
+from .fiterax import FiteraxConfig
 from .gilozen import GilozenConfig
 from .qwen2 import Qwen2Config
 
-__all__ = ["BotulornConfig", "ConfigError", "GilozenConfig", "ModelConfig", "Qwen2Config", "read_config_json"]
+__all__ = ["BotulornConfig", "ConfigError", "FiteraxConfig", "GilozenConfig", "ModelConfig", "Qwen2Config", "read_config_json"]

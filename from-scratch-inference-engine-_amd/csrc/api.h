@@ -42,8 +42,9 @@ int fsie_device_info(char* arch_out, int arch_len, int* n_compute_units);
 // Compute units of the current device; 0 if there is no device to ask.
 int fsie_device_compute_units(void);
 
+// out[t] = table[ids[t]] * scale, float32
 int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out, int n_tokens, int hidden,
-                   int vocab, hipStream_t stream);
+                   int vocab, float scale, hipStream_t stream);
 int fsie_rmsnorm(float* residual, const void* delta, const float* weight, void* out, const int32_t* rows,
                  int n_rows, int hidden, float eps, int dtype, int write_back, int n_parts, int total_rows,
                  hipStream_t stream);
@@ -134,7 +135,7 @@ int fsie_attention_prep(const void* proj, int64_t stride, int q_off, int k_off, 
                         int kv_heads, int dim, int vdim, int D, const float* q_weight, const float* k_weight, float eps,
                         int pairs, const float* cos_sin, const void* v_other, int64_t v_other_stride, const float* mix,
                         void* q_out, float* gate, const int32_t* slots, void* k_pool, void* v_pool, int page_size,
-                        int64_t pool_slots, int n_tokens, int dtype, hipStream_t stream);
+                        int64_t pool_slots, int n_tokens, int dtype, int q_weight_stride, hipStream_t stream);
 int fsie_gate_heads(const void* x, int D, const float* gate, void* y, int n_tokens, int heads, int vdim, int dtype,
                     hipStream_t stream);
 
@@ -178,7 +179,9 @@ int fsie_fragment_order(const void* w, void* out, int N, int K, hipStream_t stre
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
                           void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,
-                          int window, float scale, int dtype, const float* sinks, hipStream_t stream);
+                          int window, float scale, int dtype, const float* sinks, float softcap, hipStream_t stream);
+// softcap (in every attention entry point that takes it): a positive number caps the scaled scores,
+// s <- softcap * tanh(s / softcap), before the mask and the softmax; 0: scores as they are.
 // sinks (or null, in every attention entry point that takes it): float32 [n_heads]; exp(sinks[h]) is one more
 // term of the softmax denominator of every query row of head h.  It has no key and no value and is not scaled.
 // Items that leave partial records ignore it; the merge that combines them adds it once.
@@ -189,7 +192,7 @@ int fsie_attention_scalar_tile_tokens(int n_heads, int n_kv);
 int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                         const int32_t* block_tables, int max_pages, const int32_t* items, int n_items, void* out,
                         float* partials, int n_heads, int n_kv, int head_dim, int page_size, int window, float scale,
-                        int large, int waves, const float* sinks, hipStream_t stream);
+                        int large, int waves, const float* sinks, float softcap, hipStream_t stream);
 // the same for a step of one token a request, from the q/k/v product's partial sums: bias, rotation and the
 // write into the pools happen in the kernel
 int fsie_attention_mfma_qkv_ok(int head_dim, int page_size);
@@ -202,7 +205,7 @@ int fsie_attention_mfma_lds_ok(int head_dim, int page_size);
 int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                             const int32_t* block_tables, int max_pages, const int32_t* items, const int32_t* groups,
                             int n_groups, void* out, int n_heads, int n_kv, int head_dim, int page_size, int window,
-                            float scale, const float* sinks, hipStream_t stream);
+                            float scale, const float* sinks, float softcap, hipStream_t stream);
 int fsie_attention_mfma_tiles(int head_dim, int large);
 int fsie_attention_mfma_max_waves(int head_dim);
 
@@ -235,6 +238,66 @@ int fsie_attention_split_static(const void* q, int64_t q_stride, const void* k_p
 
 int fsie_sample(const float* logits, int n_rows, int vocab, const float* temperature, const int32_t* top_k,
                 const float* top_p, const double* uniform, int32_t* out, hipStream_t stream);
+
+// ---- RMS norm in groups, over a stream with up to two pending deltas ----------------------------
+// x = residual + delta_scale * (delta1 + delta2) (either delta may be null; each is [total_rows, hidden] in its own
+// type, FSIE_F32 or FSIE_BF16), written back to `residual` if write_back; the row is cut into `groups` equal
+// consecutive parts, each divided by its own sqrt(mean(part^2) + eps); out1 = that times weight1 and, if weight2 is
+// given, out2 = that times weight2 (two norms of one stream in one pass).  `rows` (or null) selects rows; the outputs
+// have n_rows rows of type out_dtype.  Sums and the stream are float32.
+int fsie_group_rmsnorm(float* residual, const void* delta1, int delta1_dtype, const void* delta2, int delta2_dtype,
+                       float delta_scale, const float* weight1, const float* weight2, void* out1, void* out2,
+                       const int32_t* rows, int n_rows, int hidden, int groups, float eps, int out_dtype, int write_back,
+                       hipStream_t stream);
+
+// ---- a short causal convolution over time, added to its input -----------------------------------
+// y[t] = x[t] + sum_j w[:, j] * x[t - taps + 1 + j] within a request, channel by channel (w [hidden][taps], float32);
+// the inputs before a portion's first token come from state[slot] [taps - 1][hidden] (float32, oldest first; zeros
+// when the request starts), which a second kernel then brings up to date with the portion's last inputs.
+// x [n_tokens][hidden] float32, y in `dtype`; q_starts [n_seqs + 1], seq_slots [n_seqs].  `state` is the slots'
+// first record: consecutive slots lie `slot_stride` floats apart (several convolutions may share a slot).
+int fsie_causal_conv(const float* x, const float* w, void* y, float* state, int64_t slot_stride, int n_slots,
+                     const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, int hidden, int taps,
+                     int dtype, hipStream_t stream);
+
+// ---- mLSTM: a matrix memory with exponential gates ------------------------------------------------
+// gates [n_tokens][2 * heads] float32 (input gate logits, then forget gate logits); per request and head the running
+// maximum m (state record's last part) is carried: i = cap tanh(gi / cap), f = logsigmoid(cap tanh(gf / cap)),
+// m_t = max(f + m_(t-1), i).  Writes coef [n_tokens][heads][4] = (exp(f + m_(t-1) - m_t), exp(i - m_t), exp(-m_t), m_t).
+// Then the memory: S_t = keep S_(t-1) + take k v^T, n_t likewise with k alone; num[t][h][:] = S_t^T q, den[t][h] = n_t . q
+// (q scaled by q_scale).  proj [n_tokens][stride] holds q (heads * dim from q_off), k (from k_off), v (heads * vdim
+// from v_off).  state [n_slots][heads][dim * vdim + dim + 4] float32: S, n, m (and three unused numbers).
+int64_t fsie_mlstm_state_floats(int dim, int vdim);
+int fsie_mlstm_scan(const void* proj, int64_t stride, int q_off, int k_off, int v_off, int dtype, const float* gates,
+                    float gate_cap, float q_scale, float* state, int n_slots, const int32_t* q_starts,
+                    const int32_t* seq_slots, int n_seqs, int n_tokens, int heads, int dim, int vdim, float* coef,
+                    float* num, float* den, hipStream_t stream);
+// y[t][h][:] = unit_rms(num / (max(|den|, exp(-m)) + 1e-6)) * weight[h][:] * sigmoid(gate[t][h][:]), y in `dtype`;
+// gate rows lie `gate_stride` values apart (columns of the fused projection)
+int fsie_mlstm_out(const float* num, const float* den, const float* coef, const void* gate, int64_t gate_stride,
+                   const float* weight, void* y, int n_tokens, int heads, int vdim, float eps, int dtype,
+                   hipStream_t stream);
+
+// ---- routed experts ----------------------------------------------------------------------------------
+// Router: logits z = x . W^T in float32 (x [n_tokens][hidden] and W [experts][hidden] in `dtype`), s = sigmoid(z); the
+// `top` experts with the largest s + correction (ties: the lower index) are chosen; their weights are their s divided
+// by the sum of the chosen s (+ 1e-20) times `scale`.  ids [n_tokens][top] int32, weights [n_tokens][top] float32.
+int fsie_moe_route(const void* x, const void* router, const float* correction, int dtype, int32_t* ids, float* weights,
+                   int n_tokens, int hidden, int experts, int top, float scale, hipStream_t stream);
+// Groups the n = n_tokens * top (token, choice) pairs by expert: order[slot] = pair (slots of one expert are
+// consecutive), slot_of[pair] = slot, and a table of row tiles of `tile_rows` slots that never cross an expert:
+// tiles [max_tiles][3] = (expert, first slot, slots), max_tiles = ceil(n / tile_rows) + experts; unused tiles have 0 slots.
+int fsie_moe_group(const int32_t* ids, int n_pairs, int experts, int tile_rows, int32_t* order, int32_t* slot_of,
+                   int32_t* tiles, int max_tiles, hipStream_t stream);
+// One product per expert over its tiles: out[slot] = epilogue(A[row(slot)] . W[expert]^T), W [experts][N][K] in `dtype`.
+// gather_div > 0: row(slot) = order[slot] / gather_div (rows of A are tokens); 0: row(slot) = slot.
+// epilogue 0: exact GELU, out in `dtype`; 1: times slot_weight[order[slot]], out float32.
+int fsie_moe_gemm(const void* a, const void* w, void* out, const int32_t* tiles, int max_tiles, const int32_t* order,
+                  int gather_div, const float* pair_weight, int N, int K, int epilogue, int dtype, int tile_rows,
+                  hipStream_t stream);
+// y[t] = sum over the token's choices, in their order, of rows[slot_of[t * top + c]]; y float32 [n_tokens][hidden]
+int fsie_moe_combine(const float* rows, const int32_t* slot_of, float* y, int n_tokens, int top, int hidden,
+                     hipStream_t stream);
 
 #ifdef __cplusplus
 }

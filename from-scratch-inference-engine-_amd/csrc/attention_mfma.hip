@@ -31,7 +31,8 @@ extern "C" int fsie_attention_mfma_tiles(int head_dim, int large) {
 extern "C" int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                                    const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
                                    void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,
-                                   int window, float scale, int large, int waves, const float* sinks, hipStream_t stream) {
+                                   int window, float scale, int large, int waves, const float* sinks, float softcap,
+                                   hipStream_t stream) {
     FSIE_REQUIRE(n_items >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
                  "attention_mfma: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
     FSIE_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
@@ -50,7 +51,7 @@ extern "C" int fsie_attention_mfma(const void* q, int64_t q_stride, const void* 
                            : hdt <= 12 ? fsie_attn::table_c(hdt, large) : fsie_attn::table_d(hdt, large);
     FSIE_REQUIRE(fn != nullptr, "attention_mfma: no kernel for head_dim %d", head_dim);
     return fn(q, q_stride, k_pool, v_pool, block_tables, max_pages, items, n_items, out, partials, n_heads, n_kv,
-              page_size, window, scale, waves, sinks, stream);
+              page_size, window, scale, waves, sinks, softcap, stream);
 }
 
 // Whether fsie_attention_mfma_qkv has a kernel for these sizes.

@@ -80,6 +80,7 @@ struct QkvSums {
     int64_t pool_slots;
     int n_parts, width;
     const float* sinks;    // [n_heads] or null: exp(sink) joins every row's denominator (any variant)
+    float softcap;         // > 0: the scaled scores become softcap * tanh(score / softcap) (any variant); 0: as they are
 };
 
 // Element d of a head after the rotation of the pairs (i, i + HD / 2) by the angles whose
@@ -171,6 +172,10 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     const int G = lane >> 4;  // lane group: which 4 (or 8) of the reduction indices this lane holds
     const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
     const float scale2 = scale * kLog2e;  // scores in units of log2 e: exp() becomes exp2()
+    // capped scores: softcap * tanh(product * scale / softcap), in the same units
+    const bool capped = f.softcap > 0.f;
+    const float cap2 = f.softcap * kLog2e, cap_in = capped ? scale / f.softcap : 0.f;
+    auto scaled = [&](float product) { return capped ? cap2 * tanh_by_exp(product * cap_in) : product * scale2; };
 
     // LDS: the accumulators that the waves after the first hand over at the end; before that, in
     // the QKV variant, the heads added up from the sums (up to 16 of queries, a key, a value) and
@@ -417,7 +422,7 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
             if (full) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    sv[i] = st[i >> 2][i & 3] * scale2;
+                    sv[i] = scaled(st[i >> 2][i & 3]);
                     m_loc = fmaxf(m_loc, sv[i]);
                 }
             } else {
@@ -429,7 +434,7 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
                         const bool in_range = kept_block ? key < prefix_end : (key >= key_begin && key < key_end);
                         const bool vis = rvalid[nt] && in_range && key <= rpos[nt] &&
                                          (window <= 0 || key > rpos[nt] - window || key < keep);
-                        sv[t * 4 + r] = vis ? st[t][r] * scale2 : -INFINITY;
+                        sv[t * 4 + r] = vis ? scaled(st[t][r]) : -INFINITY;
                         m_loc = fmaxf(m_loc, sv[t * 4 + r]);
                     }
             }
@@ -705,10 +710,11 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
 template <int HDT, int NT>
 int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool, const int32_t* block_tables,
            int max_pages, const int32_t* items, int n_items, void* out, float* partials, int n_heads, int n_kv,
-           int page_size, int window, float scale, int waves, const float* sinks, hipStream_t stream) {
+           int page_size, int window, float scale, int waves, const float* sinks, float softcap, hipStream_t stream) {
     constexpr int MAXW = NT == 1 ? max_waves<HDT>() : 4;
     QkvSums only_sinks{};
     only_sinks.sinks = sinks;
+    only_sinks.softcap = softcap;
     const int group = n_heads / n_kv;
     const int rows = 16 * NT;
     const int gh = group < rows ? group : rows;
@@ -765,6 +771,6 @@ typedef int (*LaunchQkvFn)(const QkvSums&, const void*, const void*, const int32
                            float*, int, int, int, int, float, int, hipStream_t);
 
 typedef int (*LaunchFn)(const void*, int64_t, const void*, const void*, const int32_t*, int, const int32_t*, int, void*,
-                        float*, int, int, int, int, float, int, const float*, hipStream_t);
+                        float*, int, int, int, int, float, int, const float*, float, hipStream_t);
 
 }  // namespace fsie_attn

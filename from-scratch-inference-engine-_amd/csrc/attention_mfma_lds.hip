@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, const int32_t* __restrict__ groups, bf16_t* __restrict__ out, int n_heads,
     int n_kv, int page_size_arg, int window, float scale, int gh, int head_chunks, int n_groups, int n_y,
-    int units_per_die, const float* __restrict__ sinks) {
+    int units_per_die, const float* __restrict__ sinks, float softcap) {
     constexpr int HD = HDT * 16;
     const int page_size = PS > 0 ? PS : page_size_arg;
     constexpr int S32 = HDT / 2;       // 32-wide steps over the head dimension
@@ -150,6 +150,10 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const int seq_wg = items[static_cast<int64_t>(first) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_SEQ];
     const int32_t* table = block_tables + static_cast<int64_t>(seq_wg) * max_pages;
     const float scale2 = scale * kLog2e;
+    // capped scores: a product p becomes (softcap / scale) * tanh(p * scale / softcap), still in the products' units
+    const bool capped = softcap > 0.f;
+    const float cap_in = capped ? scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
+    auto score_of = [&](float product) { return capped ? cap_out * tanh_by_exp(product * cap_in) : product; };
 
     // ---- this wave's queries (B operands)
     bool rvalid[NT];
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
             for (int nt = 0; nt < NT; ++nt) {
                 if (full) {
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) sv[h][nt][i] = st[h][nt][i >> 2][i & 3];
+                    for (int i = 0; i < 8; ++i) sv[h][nt][i] = score_of(st[h][nt][i >> 2][i & 3]);
                 } else {
 #pragma unroll
                     for (int tt = 0; tt < 2; ++tt)
@@ -327,7 +331,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
                                                              : ((key >= key_begin && key < key_end) || key < kept_in_range);
                             const bool vis = rvalid[nt] && in_range && key <= rpos[nt] &&
                                              (window <= 0 || key > rpos[nt] - window || key < keep);
-                            sv[h][nt][tt * 4 + r] = vis ? st[h][nt][tt][r] : -INFINITY;
+                            sv[h][nt][tt * 4 + r] = vis ? score_of(st[h][nt][tt][r]) : -INFINITY;
                         }
                 }
 #pragma unroll
@@ -442,7 +446,8 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
 template <int HDT, int PS>
 int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf16_t* v_pool,
                const int32_t* block_tables, int max_pages, const int32_t* items, const int32_t* groups, int n_groups,
-               bf16_t* out, int n_heads, int n_kv, int page_size, int window, float scale, const float* sinks, hipStream_t stream) {
+               bf16_t* out, int n_heads, int n_kv, int page_size, int window, float scale, const float* sinks, float softcap,
+               hipStream_t stream) {
     const int group = n_heads / n_kv;
     const int gh = group < 32 ? group : 32;
     const int head_chunks = (group + gh - 1) / gh;
@@ -453,7 +458,7 @@ int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf
     attention_mfma_lds_kernel<HDT, PS><<<grid, kLdsThreads, 0, stream>>>(q, q_stride, k_pool, v_pool, block_tables, max_pages,
                                                                      items, groups, out, n_heads, n_kv, page_size,
                                                                      window, scale, gh, head_chunks, n_groups,
-                                                                     by_die ? ys : 0, max(1, fsie_compute_units() / 8), sinks);
+                                                                     by_die ? ys : 0, max(1, fsie_compute_units() / 8), sinks, softcap);
     FSIE_CHECK_LAUNCH("attention_mfma_lds");
     return 0;
 }
@@ -474,7 +479,8 @@ extern "C" int fsie_attention_mfma_lds_ok(int head_dim, int page_size) {
 extern "C" int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                                        const int32_t* block_tables, int max_pages, const int32_t* items,
                                        const int32_t* groups, int n_groups, void* out, int n_heads, int n_kv,
-                                       int head_dim, int page_size, int window, float scale, const float* sinks, hipStream_t stream) {
+                                       int head_dim, int page_size, int window, float scale, const float* sinks, float softcap,
+                                       hipStream_t stream) {
     FSIE_REQUIRE(n_groups >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
                  "attention_mfma_lds: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
     FSIE_REQUIRE(fsie_attention_mfma_lds_ok(head_dim, page_size),
@@ -492,9 +498,9 @@ extern "C" int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const vo
     case H:                                                                                                        \
         return page_size == 16                                                                                     \
                    ? fsie_attn::launch_lds<H, 16>(qq, q_stride, kk, vv, block_tables, max_pages, items, groups,    \
-                                                  n_groups, oo, n_heads, n_kv, page_size, window, scale, sinks, stream) \
+                                                  n_groups, oo, n_heads, n_kv, page_size, window, scale, sinks, softcap, stream) \
                    : fsie_attn::launch_lds<H, 0>(qq, q_stride, kk, vv, block_tables, max_pages, items, groups,     \
-                                                 n_groups, oo, n_heads, n_kv, page_size, window, scale, sinks, stream)
+                                                 n_groups, oo, n_heads, n_kv, page_size, window, scale, sinks, softcap, stream)
     switch (head_dim / 16) {
         FSIE_LDS_CASE(2);
         FSIE_LDS_CASE(4);

@@ -3,7 +3,8 @@
 //
 // proj [tokens][stride] holds of every token q (heads * dim from q_off), k (kv_heads * dim from k_off),
 // v (kv_heads * vdim from v_off) and, optionally, one gate logit a head (from g_off).  Per token:
-//   q, k heads: RMS norm over dim with a weight shared by the heads (q_weight / k_weight, or none), then the
+//   q, k heads: RMS norm over dim with a weight shared by the heads (q_weight / k_weight, or none; the query heads'
+//               weights may also differ: head h then takes q_weight + h * q_weight_stride), then the
 //               first 2 * pairs values turned, value i with value i + pairs, by the step's cosines and sines
 //               cos_sin [tokens][pairs][2]; all of it float32
 //   v:          (1 - mix) v + mix * v_other where another layer's values of the same token are given
@@ -66,7 +67,8 @@ __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
     int vdim, int D, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps, int pairs,
     const float2* __restrict__ cos_sin, const T* __restrict__ v_other, int64_t v_other_stride, const float* __restrict__ mix,
     T* __restrict__ q_out, float* __restrict__ gate, const int32_t* __restrict__ slots, T* __restrict__ k_pool,
-    T* __restrict__ v_pool, int page_size, int64_t pool_slots, int values_elsewhere, int L, int head_blocks) {
+    T* __restrict__ v_pool, int page_size, int64_t pool_slots, int values_elsewhere, int L, int head_blocks,
+    int q_weight_stride) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int side = 64 / L;  // heads side by side in a pass
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
     const int n_heads_all = heads + kv_heads;
     // where head `unit` is read from, which weight it takes and where it goes (null: nowhere)
     auto source = [&](int unit) { return row + (unit < heads ? q_off + unit * dim : k_off + (unit - heads) * dim); };
-    auto weight = [&](int unit) { return unit < heads ? q_weight : k_weight; };
+    auto weight = [&](int unit) { return unit < heads ? (q_weight ? q_weight + unit * q_weight_stride : nullptr) : k_weight; };
     auto target = [&](int unit) -> T* {
         if (unit < heads) return q_out + (static_cast<int64_t>(t) * heads + unit) * D;
         return store ? k_pool + ((page * kv_heads + (unit - heads)) * page_size + off) * D : nullptr;
@@ -245,7 +247,7 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
                                    float eps, int pairs, const float* cos_sin, const void* v_other, int64_t v_other_stride,
                                    const float* mix, void* q_out, float* gate, const int32_t* slots, void* k_pool,
                                    void* v_pool, int page_size, int64_t pool_slots, int n_tokens, int dtype,
-                                   hipStream_t stream) {
+                                   int q_weight_stride, hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0 && D >= dim && D >= vdim,
                  "attention_prep: bad sizes heads=%d kv=%d dim=%d vdim=%d D=%d", heads, kv_heads, dim, vdim, D);
     FSIE_REQUIRE(pairs >= 0 && 2 * pairs <= dim && (pairs == 0 || cos_sin), "attention_prep: %d rotated pairs in heads of %d",
@@ -257,7 +259,8 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
     if (n_tokens == 0) return 0;
     const auto mult4 = [](int64_t v) { return (v & 3) == 0; };
     const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    const bool vec = D <= 256 && mult4(stride) && mult4(q_off) && mult4(k_off) && mult4(dim) && mult4(D) && mult4(pairs) && al16(proj) &&
+    FSIE_REQUIRE(q_weight_stride >= 0, "attention_prep: bad stride of the query heads' weights");
+    const bool vec = D <= 256 && mult4(q_weight_stride) && mult4(stride) && mult4(q_off) && mult4(k_off) && mult4(dim) && mult4(D) && mult4(pairs) && al16(proj) &&
                      al16(q_out) && al16(k_pool) && al16(q_weight) && al16(k_weight) && al16(cos_sin);
     // portions of prompts in bfloat16: the values go through the kernel that writes eight slots at once
     const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= kPortionTokens && al16(v_pool)) ? 1 : 0;
@@ -276,7 +279,7 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
         static_cast<const T*>(proj), stride, q_off, k_off, v_off, g_off, heads, kv_heads, dim, vdim, D, q_weight, k_weight, \
         eps, pairs, reinterpret_cast<const float2*>(cos_sin), static_cast<const T*>(v_other), v_other_stride, mix,       \
         static_cast<T*>(q_out), gate, slots, static_cast<T*>(k_pool), static_cast<T*>(v_pool), page_size, pool_slots,   \
-        values_elsewhere, lanes, head_blocks)
+        values_elsewhere, lanes, head_blocks, q_weight_stride)
 #define FSIE_PREP_V(T, V) \
     if (hpw == 4) FSIE_PREP_H(T, V, 4); else FSIE_PREP_H(T, V, 1)
 #define FSIE_PREP(T) \

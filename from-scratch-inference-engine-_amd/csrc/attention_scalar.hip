@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_pages, const int32_t* __restrict__ items,
     T* __restrict__ out, float* __restrict__ partials, int n_heads, int n_kv, int hd, int page_size,
-    int window, float scale, int gh, int head_chunks, const float* __restrict__ sinks) {
+    int window, float scale, int gh, int head_chunks, const float* __restrict__ sinks, float softcap) {
     extern __shared__ float lds[];
     float* qs = lds;                          // [kRows][hd]
     float* kv = qs + kRows * hd;              // [kKeys][hd + 1]
@@ -159,6 +159,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
                 float dot = 0.f;
                 for (int d = 0; d < hd; ++d) dot = fmaf(qr[d], kr[d], dot);
                 s = dot * scale;
+                if (softcap > 0.f) s = softcap * tanhf(s / softcap);  // capped scores: softcap * tanh(s / softcap)
             }
             const float m_new = fmaxf(m_run[p], half_wave_max(s));
             const float pe = (s == -INFINITY) ? 0.f : expf(s - m_new);
@@ -394,7 +395,7 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
                                      const int32_t* block_tables, int max_pages, const int32_t* items,
                                      int n_items, void* out, float* partials, int n_heads, int n_kv,
                                      int head_dim, int page_size, int window, float scale, int dtype,
-                                     const float* sinks, hipStream_t stream) {
+                                     const float* sinks, float softcap, hipStream_t stream) {
     FSIE_REQUIRE(n_items >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
                  "attention: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
     FSIE_REQUIRE(head_dim > 0 && head_dim <= 32 * kMaxChunksWide, "attention: head_dim %d must be in 1..%d",
@@ -422,7 +423,7 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
         kernel<<<grid, 256, lds, stream>>>(static_cast<const T*>(q), q_stride, static_cast<const T*>(k_pool),        \
                                            static_cast<const T*>(v_pool), block_tables, max_pages, items,            \
                                            static_cast<T*>(out), partials, n_heads, n_kv, head_dim, page_size, window, \
-                                           scale, gh, head_chunks, sinks);                                           \
+                                           scale, gh, head_chunks, sinks, softcap);                                  \
     } while (0)
 #define FSIE_SCALAR_ATTENTION_OF(T)                                          \
     if (wide) {                                                              \

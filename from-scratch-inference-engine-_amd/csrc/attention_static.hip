@@ -102,9 +102,9 @@ extern "C" int fsie_attention_split_static(const void* q, int64_t q_stride, cons
     // nothing has to start at zero: an item writes the whole record of every slot that a merge
     // reads, and a merge reads no other slot
     int rc = mfma ? fsie_attention_mfma(q, q_stride, k_pool, v_pool, block_tables, max_pages, items_in, n_items, out,
-                                        partials, n_heads, n_kv, head_dim, page_size, window, scale, 0, waves, nullptr, stream)
+                                        partials, n_heads, n_kv, head_dim, page_size, window, scale, 0, waves, nullptr, 0.f, stream)
                   : fsie_attention_scalar(q, q_stride, k_pool, v_pool, block_tables, max_pages, items_in, n_items, out,
-                                          partials, n_heads, n_kv, head_dim, page_size, window, scale, dtype, nullptr, stream);
+                                          partials, n_heads, n_kv, head_dim, page_size, window, scale, dtype, nullptr, 0.f, stream);
     if (rc) return rc;
     return fsie_attention_merge(partials, merges_in, n_merges, out, n_heads, head_dim, dtype, nullptr, stream);
 }

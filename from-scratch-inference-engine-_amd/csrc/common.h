@@ -62,6 +62,13 @@ __device__ __forceinline__ float gate_act(float g, int act) {
     return g / (1.0f + expf(-g));
 }
 
+// tanh through one exponential, 1 - 2 / (exp(2x) + 1): within a few float32 roundings of 1 in absolute terms,
+// right at both ends (exp overflows to infinity: 1; underflows to 0: -1); for score caps in kernels that
+// work in bfloat16 anyway.  Float32 paths call tanhf.
+__device__ __forceinline__ float tanh_by_exp(float x) {
+    return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f);
+}
+
 // ---- reductions over a 64-lane wave ------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

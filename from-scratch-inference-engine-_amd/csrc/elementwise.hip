@@ -13,7 +13,7 @@ constexpr int kWideNormRows = 128;  // up to so many rows (half the device's uni
 // host refuses such ids before the launch.
 template <typename T>
 __global__ void embedding_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
-                                 float* __restrict__ out, int hidden, int vocab) {
+                                 float* __restrict__ out, int hidden, int vocab, float scale) {
     const int t = blockIdx.x;
     const int id = ids[t];
     float* dst = out + static_cast<int64_t>(t) * hidden;
@@ -22,7 +22,7 @@ __global__ void embedding_kernel(const T* __restrict__ table, const int32_t* __r
         return;
     }
     const T* src = table + static_cast<int64_t>(id) * hidden;
-    for (int j = threadIdx.x; j < hidden; j += blockDim.x) dst[j] = to_float(src[j]);
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) dst[j] = to_float(src[j]) * scale;
 }
 
 // One block per output row r; source row = rows ? rows[r] : r.
@@ -93,13 +93,14 @@ struct Pack4<bf16_t> {
 // four elements per thread, grid = (tokens, quads / threads): no loop, one load per thread
 template <typename T>
 __global__ void embedding_vec_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
-                                     float* __restrict__ out, int hidden, int vocab) {
+                                     float* __restrict__ out, int hidden, int vocab, float scale) {
     const int t = blockIdx.x;
     const int j = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
     if (j >= hidden) return;
     const int id = ids[t];
     const bool ok = id >= 0 && id < vocab;
-    const float4 v = Pack4<T>::load(table + static_cast<int64_t>(ok ? id : 0) * hidden + j);
+    float4 v = Pack4<T>::load(table + static_cast<int64_t>(ok ? id : 0) * hidden + j);
+    v = float4{v.x * scale, v.y * scale, v.z * scale, v.w * scale};  // (times 1 changes no bit)
     Pack4<float>::store(out + static_cast<int64_t>(t) * hidden + j, ok ? v : float4{0.f, 0.f, 0.f, 0.f});
 }
 
@@ -451,7 +452,7 @@ extern "C" int fsie_rmsnorm_plain(const void* x, int64_t x_stride, const float* 
 }
 
 extern "C" int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out,
-                              int n_tokens, int hidden, int vocab, hipStream_t stream) {
+                              int n_tokens, int hidden, int vocab, float scale, hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes T=%d H=%d V=%d",
                  n_tokens, hidden, vocab);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "embedding: unknown dtype %d", dtype);
@@ -459,11 +460,11 @@ extern "C" int fsie_embedding(const void* table, int dtype, const int32_t* ids, 
     const bool vec = hidden % 4 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
     const dim3 vgrid(n_tokens, static_cast<unsigned>(ceil_div64(hidden / 4, kThreads)));
     if (dtype == FSIE_F32) {
-        if (vec) embedding_vec_kernel<float><<<vgrid, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
-        else embedding_kernel<float><<<n_tokens, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
+        if (vec) embedding_vec_kernel<float><<<vgrid, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab, scale);
+        else embedding_kernel<float><<<n_tokens, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab, scale);
     } else {
-        if (vec) embedding_vec_kernel<bf16_t><<<vgrid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab);
-        else embedding_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab);
+        if (vec) embedding_vec_kernel<bf16_t><<<vgrid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab, scale);
+        else embedding_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab, scale);
     }
     FSIE_CHECK_LAUNCH("embedding");
     return 0;

@@ -1,0 +1,189 @@
+// RMS norm in groups over the residual stream, fused with the residual sum of up to two pending deltas, and the
+// short causal convolution that a layer may put in front of what its sublayers read.
+//
+// group_rmsnorm: one workgroup a row.  x = residual + delta_scale * (delta1 + delta2) goes to LDS (and back to the
+// stream); the row is `groups` equal consecutive parts, a wave takes a part at a time and leaves
+// 1 / sqrt(mean(part^2) + eps) in LDS; then every thread writes x * that * weight, for one or two weights.
+//
+// causal_conv: y[t] = x[t] + sum_j w[:, j] x[t - taps + 1 + j]; inputs before a portion's start come from the
+// request's state (the last taps - 1 inputs, oldest first).  A second kernel stores the new last inputs after
+// every row has been written, so no block reads a state that another has already replaced.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxGroups = 256;
+
+template <typename D>
+__device__ __forceinline__ float delta_at(const D* d, int64_t i) { return d ? to_float(d[i]) : 0.f; }
+
+template <typename T, typename D1, typename D2>
+__global__ __launch_bounds__(kThreads) void group_rmsnorm_kernel(
+    float* __restrict__ residual, const D1* __restrict__ delta1, const D2* __restrict__ delta2, float delta_scale,
+    const float* __restrict__ weight1, const float* __restrict__ weight2, T* __restrict__ out1, T* __restrict__ out2,
+    const int32_t* __restrict__ rows, int hidden, int groups, float eps, int write_back) {
+    extern __shared__ float lds[];
+    float* xs = lds;               // [hidden]
+    float* inv = lds + hidden;     // [groups]
+    const int r = blockIdx.x;
+    const int64_t row = rows ? rows[r] : r;
+    float* res = residual + row * hidden;
+    const bool has_delta = delta1 || delta2;
+    for (int j = threadIdx.x; j < hidden; j += kThreads) {
+        float v = res[j];
+        if (has_delta) {
+            // the two sublayers' outputs first, then the factor, then the stream: one order for every caller
+            const float d = delta_at(delta1, row * hidden + j) + delta_at(delta2, row * hidden + j);
+            v = fmaf(delta_scale, d, v);
+            if (write_back) res[j] = v;
+        }
+        xs[j] = v;
+    }
+    __syncthreads();
+    const int part = hidden / groups;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int g = wave; g < groups; g += kThreads / 64) {
+        const float* p = xs + g * part;
+        float sum = 0.f;
+        for (int j = lane; j < part; j += 64) sum = fmaf(p[j], p[j], sum);
+        sum = wave_sum(sum);
+        if (lane == 0) inv[g] = 1.0f / sqrtf(sum / static_cast<float>(part) + eps);
+    }
+    __syncthreads();
+    T* o1 = out1 + static_cast<int64_t>(r) * hidden;
+    T* o2 = out2 ? out2 + static_cast<int64_t>(r) * hidden : nullptr;
+    for (int j = threadIdx.x; j < hidden; j += kThreads) {
+        const float n = xs[j] * inv[j / part];
+        o1[j] = from_float<T>(n * weight1[j]);
+        if (o2) o2[j] = from_float<T>(n * weight2[j]);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void causal_conv_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                               T* __restrict__ y, const float* __restrict__ state,
+                                                               int64_t slot_stride, int n_slots,
+                                                               const int32_t* __restrict__ q_starts,
+                                                               const int32_t* __restrict__ seq_slots, int n_seqs, int hidden,
+                                                               int taps) {
+    __shared__ int s_info[2];
+    const int t = blockIdx.x;
+    if (threadIdx.x == 0) {
+        // the request of this row: the last one whose first row is not beyond it
+        int lo = 0, hi = n_seqs - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (q_starts[mid] <= t) lo = mid; else hi = mid - 1;
+        }
+        const int slot = seq_slots[lo];
+        s_info[0] = q_starts[lo];
+        s_info[1] = (slot >= 0 && slot < n_slots) ? slot : -1;
+    }
+    __syncthreads();
+    const int first = s_info[0], slot = s_info[1];
+    const float* st = slot >= 0 ? state + slot * slot_stride : nullptr;
+    for (int c = threadIdx.x; c < hidden; c += kThreads) {
+        const float here = x[static_cast<int64_t>(t) * hidden + c];
+        float acc = here;
+        for (int j = 0; j < taps; ++j) {
+            const int back = taps - 1 - j;  // how many tokens before this one
+            const int src = t - back;
+            float v;
+            if (src >= first) v = back ? x[static_cast<int64_t>(src) * hidden + c] : here;
+            else v = st ? st[static_cast<int64_t>(taps - 1 - (first - src)) * hidden + c] : 0.f;  // state row taps-1-k = k tokens before the portion
+            acc = fmaf(w[c * taps + j], v, acc);
+        }
+        y[static_cast<int64_t>(t) * hidden + c] = from_float<T>(acc);
+    }
+}
+
+// state'[i] for i in [0, taps - 1): the input (taps - 1 - i) tokens before the next portion's first token
+__global__ __launch_bounds__(kThreads) void causal_conv_store_kernel(const float* __restrict__ x, float* __restrict__ state,
+                                                                     int64_t slot_stride, int n_slots,
+                                                                     const int32_t* __restrict__ q_starts,
+                                                                     const int32_t* __restrict__ seq_slots, int hidden,
+                                                                     int taps) {
+    const int s = blockIdx.x;
+    const int slot = seq_slots[s];
+    const int first = q_starts[s], n = q_starts[s + 1] - first;
+    if (slot < 0 || slot >= n_slots || n <= 0) return;
+    float* st = state + slot * slot_stride;
+    const int keep = taps - 1;
+    for (int c = threadIdx.x; c < hidden; c += kThreads) {
+        // a thread owns its channel: old rows are read before they are overwritten (ascending i reads row i + n >= i)
+        for (int i = 0; i < keep; ++i) {
+            const int back = keep - i;  // tokens before the next portion's start
+            float v;
+            if (back <= n) v = x[static_cast<int64_t>(first + n - back) * hidden + c];
+            else v = st[static_cast<int64_t>(i + n) * hidden + c];  // still an input of an earlier step: row i + n of the old state
+            st[static_cast<int64_t>(i) * hidden + c] = v;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int fsie_group_rmsnorm(float* residual, const void* delta1, int delta1_dtype, const void* delta2, int delta2_dtype,
+                                  float delta_scale, const float* weight1, const float* weight2, void* out1, void* out2,
+                                  const int32_t* rows, int n_rows, int hidden, int groups, float eps, int out_dtype,
+                                  int write_back, hipStream_t stream) {
+    FSIE_REQUIRE(n_rows >= 0 && hidden > 0 && groups > 0 && groups <= kMaxGroups && hidden % groups == 0,
+                 "group_rmsnorm: %d values do not make %d equal groups (at most %d)", hidden, groups, kMaxGroups);
+    FSIE_REQUIRE(residual && weight1 && out1 && (!weight2) == (!out2), "group_rmsnorm: missing operand");
+    FSIE_REQUIRE(out_dtype == FSIE_F32 || out_dtype == FSIE_BF16, "group_rmsnorm: unknown dtype %d", out_dtype);
+    FSIE_REQUIRE((!delta1 || delta1_dtype == FSIE_F32 || delta1_dtype == FSIE_BF16) &&
+                     (!delta2 || delta2_dtype == FSIE_F32 || delta2_dtype == FSIE_BF16), "group_rmsnorm: unknown delta dtype");
+    FSIE_REQUIRE(!(rows && write_back), "group_rmsnorm: chosen rows are not written back");
+    if (n_rows == 0) return 0;
+    const size_t lds = sizeof(float) * (static_cast<size_t>(hidden) + groups);
+    FSIE_REQUIRE(lds <= 64 * 1024, "group_rmsnorm: rows of %d values are more than the kernel holds", hidden);
+#define FSIE_GN(T, D1, D2)                                                                                              \
+    do {                                                                                                                \
+        auto kernel = group_rmsnorm_kernel<T, D1, D2>;                                                                  \
+        if (lds > 48 * 1024) {                                                                                          \
+            const hipError_t ok = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                            \
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+            FSIE_REQUIRE(ok == hipSuccess, "group_rmsnorm: %zu bytes of shared memory: %s", lds, hipGetErrorString(ok)); \
+        }                                                                                                               \
+        kernel<<<n_rows, kThreads, lds, stream>>>(residual, static_cast<const D1*>(delta1), static_cast<const D2*>(delta2), \
+                                                  delta_scale, weight1, weight2, static_cast<T*>(out1),                 \
+                                                  static_cast<T*>(out2), rows, hidden, groups, eps, write_back);        \
+    } while (0)
+#define FSIE_GN_D(T)                                                                       \
+    if (delta1_dtype == FSIE_F32 && delta2_dtype == FSIE_F32) FSIE_GN(T, float, float);    \
+    else if (delta1_dtype == FSIE_F32) FSIE_GN(T, float, bf16_t);                          \
+    else if (delta2_dtype == FSIE_F32) FSIE_GN(T, bf16_t, float);                          \
+    else FSIE_GN(T, bf16_t, bf16_t)
+    if (!delta1) delta1_dtype = FSIE_F32;
+    if (!delta2) delta2_dtype = FSIE_F32;
+    if (out_dtype == FSIE_F32) { FSIE_GN_D(float); } else { FSIE_GN_D(bf16_t); }
+#undef FSIE_GN_D
+#undef FSIE_GN
+    FSIE_CHECK_LAUNCH("group_rmsnorm");
+    return 0;
+}
+
+extern "C" int fsie_causal_conv(const float* x, const float* w, void* y, float* state, int64_t slot_stride, int n_slots,
+                                const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, int hidden,
+                                int taps, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && hidden > 0 && taps >= 1 && n_slots > 0,
+                 "causal_conv: bad sizes T=%d requests=%d hidden=%d taps=%d", n_tokens, n_seqs, hidden, taps);
+    FSIE_REQUIRE(x && w && y && q_starts && seq_slots && (taps == 1 || state), "causal_conv: missing operand");
+    FSIE_REQUIRE(slot_stride >= static_cast<int64_t>(taps - 1) * hidden, "causal_conv: slots closer than a state is long");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "causal_conv: unknown dtype %d", dtype);
+    if (n_tokens == 0 || n_seqs == 0) return 0;
+    if (dtype == FSIE_F32)
+        causal_conv_kernel<float><<<n_tokens, kThreads, 0, stream>>>(x, w, static_cast<float*>(y), state, slot_stride, n_slots,
+                                                                     q_starts, seq_slots, n_seqs, hidden, taps);
+    else
+        causal_conv_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(x, w, static_cast<bf16_t*>(y), state, slot_stride, n_slots,
+                                                                      q_starts, seq_slots, n_seqs, hidden, taps);
+    FSIE_CHECK_LAUNCH("causal_conv");
+    if (taps > 1) {
+        causal_conv_store_kernel<<<n_seqs, kThreads, 0, stream>>>(x, state, slot_stride, n_slots, q_starts, seq_slots, hidden, taps);
+        FSIE_CHECK_LAUNCH("causal_conv_store");
+    }
+    return 0;
+}

@@ -1,0 +1,311 @@
+// Routed experts: the router, the grouping of (token, choice) pairs by expert, one product per expert over tiles
+// of its rows, and the weighted sum of a token's chosen experts.
+//
+//   route    a wave a token: float32 logits against every expert's row, sigmoid, the `top` largest of
+//            score + correction (ties to the lower index), weights = chosen scores / their sum * scale
+//   group    one workgroup: counts per expert, starts, a slot for every pair (pairs of one expert keep the order
+//            of the pairs), and the table of row tiles (expert, first slot, slots) that never cross an expert
+//   gemm     a wave per 16 slots x 64 outputs of one expert's matrix on the matrix cores: bfloat16 operands
+//            (mfma 16x16x32) or true float32 ones (mfma 16x16x4); both operands run along K in memory, which is
+//            the order the instruction wants; rows are gathered through the order table; the epilogue is the exact
+//            GELU (up) or the pair's routing weight (down, float32 result)
+//   combine  a token's rows added in the order of its choices, float32
+// Nothing here waits for the host: the tile table has a fixed worst-case length and unused tiles are empty.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kTileRows = 16;
+constexpr int kMaxExperts = 256;
+constexpr int kMaxTop = 16;
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router,
+                                                        const float* __restrict__ correction, int32_t* __restrict__ ids,
+                                                        float* __restrict__ weights, int n_tokens, int hidden, int experts,
+                                                        int top, float scale) {
+    __shared__ float s_score[4][kMaxExperts];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + wave;
+    const bool live = t < n_tokens;
+    const T* row = x + static_cast<int64_t>(live ? t : 0) * hidden;
+    float* score = s_score[wave];
+    for (int e = 0; e < experts && live; ++e) {
+        const T* w = router + static_cast<int64_t>(e) * hidden;
+        float z = 0.f;
+        for (int j = lane; j < hidden; j += 64) z = fmaf(to_float(row[j]), to_float(w[j]), z);
+        z = wave_sum(z);
+        if (lane == 0) score[e] = 1.0f / (1.0f + expf(-z));
+    }
+    __syncthreads();
+    if (!live) return;
+    // every lane walks the same choice (a few experts, a few picks): no exchange needed
+    int picked[kMaxTop];
+    float chosen[kMaxTop];
+    float total = 0.f;
+    for (int c = 0; c < top; ++c) {
+        int best = -1;
+        float best_v = -INFINITY;
+        for (int e = 0; e < experts; ++e) {
+            bool taken = false;
+            for (int p = 0; p < c; ++p) taken = taken || picked[p] == e;
+            const float v = score[e] + correction[e];
+            if (!taken && (best < 0 || v > best_v)) best = e, best_v = v;
+        }
+        picked[c] = best;
+        chosen[c] = score[best];
+        total += chosen[c];
+    }
+    if (lane < top) {
+        float mine = 0.f;
+        int id = 0;
+        for (int c = 0; c < top; ++c)
+            if (c == lane) mine = chosen[c], id = picked[c];
+        ids[static_cast<int64_t>(t) * top + lane] = id;
+        weights[static_cast<int64_t>(t) * top + lane] = mine / (total + 1e-20f) * scale;
+    }
+}
+
+// one workgroup of 1024 threads
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restrict__ ids, int n_pairs, int experts,
+                                                         int tile_rows, int32_t* __restrict__ order,
+                                                         int32_t* __restrict__ slot_of, int32_t* __restrict__ tiles,
+                                                         int max_tiles) {
+    __shared__ int s_count[kMaxExperts];
+    __shared__ int s_start[kMaxExperts + 1];
+    __shared__ int s_tile0[kMaxExperts + 1];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < experts; e += blockDim.x) s_count[e] = 0;
+    __syncthreads();
+    // thread i takes the pairs [i * chunk, (i + 1) * chunk): a pair's place among its expert's pairs is the pairs of
+    // that expert before it, so the grouping is the same whatever the hardware does first
+    const int chunk = (n_pairs + blockDim.x - 1) / blockDim.x;
+    const int lo = min(n_pairs, tid * chunk), hi = min(n_pairs, lo + chunk);
+    // pass 1: counts (an expert id outside the table is counted as expert 0; the router never makes one)
+    for (int p = lo; p < hi; ++p) {
+        int e = ids[p];
+        e = (e < 0 || e >= experts) ? 0 : e;
+        atomicAdd(&s_count[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int at = 0, tile = 0;
+        for (int e = 0; e < experts; ++e) {
+            s_start[e] = at;
+            s_tile0[e] = tile;
+            at += s_count[e];
+            tile += (s_count[e] + tile_rows - 1) / tile_rows;
+        }
+        s_start[experts] = at;
+        s_tile0[experts] = tile;
+    }
+    __syncthreads();
+    // the tile table
+    for (int i = tid; i < max_tiles; i += blockDim.x) {
+        int e = 0;
+        while (e < experts && s_tile0[e + 1] <= i) ++e;
+        int32_t* tl = tiles + 3 * i;
+        if (e >= experts) {
+            tl[0] = 0, tl[1] = 0, tl[2] = 0;
+        } else {
+            const int first = s_start[e] + (i - s_tile0[e]) * tile_rows;
+            tl[0] = e, tl[1] = first, tl[2] = min(tile_rows, s_start[e + 1] - first);
+        }
+    }
+    // pass 2: a pair's slot = its expert's start + the pairs of that expert before it.  An expert at a time: the
+    // threads' counts of it, an exclusive scan over the threads (in LDS), then the slots.
+    __shared__ int s_scan[1024];
+    for (int e = 0; e < experts; ++e) {
+        if (s_count[e] == 0) continue;  // (the same for all threads)
+        int mine = 0;
+        for (int p = lo; p < hi; ++p) {
+            int id = ids[p];
+            id = (id < 0 || id >= experts) ? 0 : id;
+            mine += id == e;
+        }
+        s_scan[tid] = mine;
+        __syncthreads();
+        for (int off = 1; off < static_cast<int>(blockDim.x); off <<= 1) {
+            const int add = tid >= off ? s_scan[tid - off] : 0;
+            __syncthreads();
+            s_scan[tid] += add;
+            __syncthreads();
+        }
+        int at = s_start[e] + s_scan[tid] - mine;
+        for (int p = lo; p < hi; ++p) {
+            int id = ids[p];
+            id = (id < 0 || id >= experts) ? 0 : id;
+            if (id == e) {
+                order[at] = p;
+                slot_of[p] = at;
+                ++at;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
+
+// A wave: 16 slots x 64 outputs (four 16 x 16 accumulators that share the rows' fragments).  Lane l supplies, for
+// the rows' operand, row l % 16 and the values of K that its lane group (l / 16) owns, and the same of a weight row
+// for the other operand; accumulator register r of lane l is (row 4 (l / 16) + r, column l % 16).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, const T* __restrict__ w, void* __restrict__ out,
+                                                       const int32_t* __restrict__ tiles, const int32_t* __restrict__ order,
+                                                       int gather_div, const float* __restrict__ pair_weight, int N, int K,
+                                                       int epilogue) {
+    const int32_t* tl = tiles + 3 * blockIdx.x;
+    const int expert = tl[0], slot0 = tl[1], n_rows = tl[2];
+    if (n_rows <= 0) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n0 = (blockIdx.y * 4 + wave) * 64;
+    if (n0 >= N) return;
+    const int r = lane & 15, g = lane >> 4;
+    const bool row_in = r < n_rows;
+    int64_t src = slot0 + r;
+    if (row_in && gather_div > 0) src = order[slot0 + r] / gather_div;
+    const T* arow = a + (row_in ? src : 0) * K;
+    const T* wbase = w + static_cast<int64_t>(expert) * N * K;
+    const T* wrow[4];
+    bool col_in[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + 16 * j + r;
+        col_in[j] = n < N;
+        wrow[j] = wbase + static_cast<int64_t>(col_in[j] ? n : 0) * K;
+    }
+    floatx4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (sizeof(T) == 2) {
+        const bool vec = (K & 7) == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
+        for (int k0 = 0; k0 < K; k0 += 32) {
+            const int k = k0 + 8 * g;
+            union { uint4 raw; bf16x8 v; uint16_t h[8]; } fa, fb[4];
+            fa.raw = uint4{0, 0, 0, 0};
+            if (vec) {
+                if (row_in && k < K) fa.raw = *reinterpret_cast<const uint4*>(arow + k);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    fb[j].raw = uint4{0, 0, 0, 0};
+                    if (col_in[j] && k < K) fb[j].raw = *reinterpret_cast<const uint4*>(wrow[j] + k);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) fa.h[i] = (row_in && k + i < K) ? arow[k + i].bits : 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) fb[j].h[i] = (col_in[j] && k + i < K) ? wrow[j][k + i].bits : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa.v, fb[j].v, acc[j], 0, 0, 0);
+        }
+    } else {
+        // true float32 on the matrix cores: an instruction takes four values of K, one a lane group
+        for (int k0 = 0; k0 < K; k0 += 4) {
+            const int k = k0 + g;
+            const float fa = (row_in && k < K) ? to_float(arow[k]) : 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float fb = (col_in[j] && k < K) ? to_float(wrow[j][k]) : 0.f;
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa, fb, acc[j], 0, 0, 0);
+            }
+        }
+    }
+    // accumulator register i: slot row 4 g + i, output n0 + 16 j + r
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = 4 * g + i;
+        if (row >= n_rows) continue;
+        const int64_t slot = slot0 + row;
+        const float scale = epilogue == 1 ? pair_weight[order[slot]] : 1.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + 16 * j + r;
+            if (n >= N) continue;
+            const float v = acc[j][i];
+            if (epilogue == 1) static_cast<float*>(out)[slot * N + n] = v * scale;
+            else static_cast<T*>(out)[slot * N + n] = from_float<T>(gelu_erf(v));
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, const int32_t* __restrict__ slot_of,
+                                                          float* __restrict__ y, int top, int hidden) {
+    const int t = blockIdx.x;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        float sum = 0.f;
+        for (int c = 0; c < top; ++c) sum += rows[static_cast<int64_t>(slot_of[t * top + c]) * hidden + j];
+        y[static_cast<int64_t>(t) * hidden + j] = sum;
+    }
+}
+
+}  // namespace
+
+extern "C" int fsie_moe_route(const void* x, const void* router, const float* correction, int dtype, int32_t* ids,
+                              float* weights, int n_tokens, int hidden, int experts, int top, float scale,
+                              hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && hidden > 0 && experts > 0 && experts <= kMaxExperts && top > 0 && top <= experts &&
+                     top <= kMaxTop, "moe_route: bad sizes T=%d hidden=%d experts=%d (at most %d) top=%d (at most %d)",
+                 n_tokens, hidden, experts, kMaxExperts, top, kMaxTop);
+    FSIE_REQUIRE(x && router && correction && ids && weights, "moe_route: missing operand");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "moe_route: unknown dtype %d", dtype);
+    if (n_tokens == 0) return 0;
+    const unsigned grid = static_cast<unsigned>((n_tokens + 3) / 4);
+    if (dtype == FSIE_F32)
+        moe_route_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x), static_cast<const float*>(router),
+                                                          correction, ids, weights, n_tokens, hidden, experts, top, scale);
+    else
+        moe_route_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(router),
+                                                           correction, ids, weights, n_tokens, hidden, experts, top, scale);
+    FSIE_CHECK_LAUNCH("moe_route");
+    return 0;
+}
+
+extern "C" int fsie_moe_group(const int32_t* ids, int n_pairs, int experts, int tile_rows, int32_t* order, int32_t* slot_of,
+                              int32_t* tiles, int max_tiles, hipStream_t stream) {
+    FSIE_REQUIRE(n_pairs >= 0 && experts > 0 && experts <= kMaxExperts && tile_rows > 0,
+                 "moe_group: bad sizes pairs=%d experts=%d tile=%d", n_pairs, experts, tile_rows);
+    FSIE_REQUIRE(max_tiles >= (n_pairs + tile_rows - 1) / tile_rows + experts, "moe_group: the tile table is too short");
+    FSIE_REQUIRE(ids && order && slot_of && tiles, "moe_group: missing operand");
+    if (n_pairs == 0) return 0;
+    moe_group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, experts, tile_rows, order, slot_of, tiles, max_tiles);
+    FSIE_CHECK_LAUNCH("moe_group");
+    return 0;
+}
+
+extern "C" int fsie_moe_gemm(const void* a, const void* w, void* out, const int32_t* tiles, int max_tiles,
+                             const int32_t* order, int gather_div, const float* pair_weight, int N, int K, int epilogue,
+                             int dtype, int tile_rows, hipStream_t stream) {
+    FSIE_REQUIRE(max_tiles >= 0 && N > 0 && K > 0 && gather_div >= 0, "moe_gemm: bad sizes tiles=%d N=%d K=%d", max_tiles, N, K);
+    FSIE_REQUIRE(tile_rows == kTileRows, "moe_gemm: tiles of %d rows (the kernel takes %d)", tile_rows, kTileRows);
+    FSIE_REQUIRE(a && w && out && tiles && order, "moe_gemm: missing operand");
+    FSIE_REQUIRE(epilogue == 0 || (epilogue == 1 && pair_weight), "moe_gemm: unknown epilogue %d", epilogue);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "moe_gemm: unknown dtype %d", dtype);
+    if (max_tiles == 0) return 0;
+    const dim3 grid(static_cast<unsigned>(max_tiles), static_cast<unsigned>((N + 255) / 256));
+    if (dtype == FSIE_F32)
+        moe_gemm_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(a), static_cast<const float*>(w), out, tiles,
+                                                         order, gather_div, pair_weight, N, K, epilogue);
+    else
+        moe_gemm_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, tiles,
+                                                          order, gather_div, pair_weight, N, K, epilogue);
+    FSIE_CHECK_LAUNCH("moe_gemm");
+    return 0;
+}
+
+extern "C" int fsie_moe_combine(const float* rows, const int32_t* slot_of, float* y, int n_tokens, int top, int hidden,
+                                hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && top > 0 && hidden > 0, "moe_combine: bad sizes");
+    FSIE_REQUIRE(rows && slot_of && y, "moe_combine: missing operand");
+    if (n_tokens == 0) return 0;
+    moe_combine_kernel<<<n_tokens, 256, 0, stream>>>(rows, slot_of, y, top, hidden);
+    FSIE_CHECK_LAUNCH("moe_combine");
+    return 0;
+}

@@ -51,6 +51,11 @@ def _require_gpu(device) -> torch.device:
 EMBEDDING_CACHE = -1  # the cache id of what the embedding keeps (the schedule's calls count from 0)
 
 
+def block_state_cache(call: int) -> int:
+    """The cache id of what the block of schedule entry ``call`` keeps itself, beside its mixer's cache."""
+    return -2 - call
+
+
 class Model:
     def __init__(self, spec: ModelSpec, dtype, device):
         self.spec = spec
@@ -69,9 +74,17 @@ class Model:
                 need = spec.layers[call.layer].mixer.cache_need()
                 if need is not None:
                     needs[i] = need
+                # what the block itself keeps for a request (the inputs of a convolution in front of its sublayers)
+                own = getattr(spec.layers[call.layer], "state_need", lambda: None)()
+                if own is not None:
+                    if getattr(own, "per_token", True):
+                        raise TypeError("a block's own need must be a per-request one")
+                    needs[block_state_cache(i)] = own
             else:
                 if not 0 <= call.cache_of < i or spec.schedule[call.cache_of].cache_of is not None:
                     raise ValueError(f"schedule entry {i}: cache_of must name an earlier call that keeps a cache")
+                if getattr(spec.layers[call.layer], "state_need", lambda: None)() is not None:
+                    raise ValueError(f"schedule entry {i}: a block that keeps a state of its own cannot borrow a cache")
                 self.call_cache.append(call.cache_of)
         # what the embedding keeps for a request between steps (a per-request need), under an id of its own
         embedding_need = spec.embedding.cache_need()
@@ -195,7 +208,11 @@ class Model:
         for i, call in enumerate(spec.schedule):
             cid = self.call_cache[i]
             cache = storage.view(cid, ctx, writes=call.cache_of is None) if cid in self.cached_calls else None
-            spec.layers[call.layer].forward(hidden, ctx, cache)
+            own = block_state_cache(i)
+            if own in self.cached_calls:
+                spec.layers[call.layer].forward(hidden, ctx, cache, state=storage.view(own, ctx, writes=True))
+            else:
+                spec.layers[call.layer].forward(hidden, ctx, cache)
         if ctx.want_rows.shape[0] == 0:
             return torch.empty((0, spec.lm_head.vocab_size), dtype=torch.float32, device=self.device)
         normed = spec.final_norm.rows(hidden, ctx.want_rows, self.dtype)

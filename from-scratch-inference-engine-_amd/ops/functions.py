@@ -59,8 +59,8 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
-def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """float32 rows of ``table`` [V, H] at ``ids`` (int32 [T]).  The caller has checked the ids."""
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """float32 rows of ``table`` [V, H] at ``ids`` (int32 [T]), times ``scale``.  The caller has checked the ids."""
     _need(table, "embedding table", ndim=2)
     _need(ids, "embedding ids", dtype=torch.int32, ndim=1)
     v, h = table.shape
@@ -69,7 +69,7 @@ def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor
         out = torch.empty((t, h), dtype=torch.float32, device=table.device)
     _need(out, "embedding out", dtype=torch.float32, shape=(t, h))
     check(load().fsie_embedding(table.data_ptr(), dtype_code(table.dtype), ids.data_ptr(), out.data_ptr(),
-                                t, h, v, _stream()))
+                                t, h, v, float(scale), _stream()))
     return out
 
 
@@ -516,7 +516,7 @@ def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_poo
                      block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
                      partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
                      window: Optional[int], scale: float, n_query_rows: int,
-                     sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> torch.Tensor:
     """Attention of the work items over the paged cache (float32 arithmetic).  ``sinks`` (float32 [n_heads],
     here and in the other attention functions): exp(sinks[h]) is one more term of the denominator of
     head h's softmax, with no key and no value.
@@ -543,7 +543,7 @@ def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_poo
                                        block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
                                        n_items, out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim,
                                        page_size, int(window or 0), float(scale), dtype_code(q.dtype),
-                                       _sinks_ptr(sinks, n_heads), _stream()))
+                                       _sinks_ptr(sinks, n_heads), float(softcap or 0.0), _stream()))
     return out
 
 
@@ -566,7 +566,7 @@ def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
                    block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
                    partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
                    window: Optional[int], scale: float, n_query_rows: int, large: bool, waves: int = 1,
-                   sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> torch.Tensor:
     """Attention of the work items over the paged cache on the matrix cores (bfloat16; head_dim a
     multiple of 16; page size a multiple of 4).  ``items`` may be a view into a longer table.
     ``waves`` waves of a workgroup split each item's keys and combine inside the workgroup."""
@@ -590,7 +590,7 @@ def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
                                      block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(), n_items,
                                      out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim, page_size,
                                      int(window or 0), float(scale), int(large), int(waves),
-                                     _sinks_ptr(sinks, n_heads), _stream()))
+                                     _sinks_ptr(sinks, n_heads), float(softcap or 0.0), _stream()))
     return out
 
 
@@ -647,7 +647,7 @@ def attention_mfma_lds_ok(head_dim: int, page_size: int) -> bool:
 def attention_mfma_lds(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
                        block_tables: torch.Tensor, items: torch.Tensor, groups: torch.Tensor, n_groups: int,
                        out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, window: Optional[int], scale: float,
-                       n_query_rows: int, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       n_query_rows: int, sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> torch.Tensor:
     """Attention of large work items (long portions) with the keys and values of a block staged in
     LDS for four tiles at once.  ``groups`` int32 [n, 2]: index in ``items`` of a group's first
     tile and its number of tiles (1..4, consecutive tiles of one request)."""
@@ -670,7 +670,7 @@ def attention_mfma_lds(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_p
                                          block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
                                          groups.data_ptr(), n_groups, out.data_ptr(), n_heads, n_kv, head_dim,
                                          page_size, int(window or 0), float(scale), _sinks_ptr(sinks, n_heads),
-                                         _stream()))
+                                         float(softcap or 0.0), _stream()))
     return out
 
 
@@ -973,7 +973,8 @@ def attention_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off
                    k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None):
     """From the fused projection ``proj`` [T, W] (q, k, v and one gate logit a head at their column offsets): the
     queries [T, heads * padded] after the heads' RMS norm (weights float32 [dim] or None) and the rotation of their
-    first ``pairs`` pairs (i, i + pairs) by ``cos_sin`` [T, pairs, 2]; the gates' sigmoid (float32 [T, heads], or
+    first ``pairs`` pairs (i, i + pairs) by ``cos_sin`` [T, pairs, 2] (``q_weight`` may also be [heads, dim]: a weight
+    of its own for every query head); the gates' sigmoid (float32 [T, heads], or
     None); and, if pools are given, keys (normed, rotated) and values written at ``slots``, the values mixed with
     ``v_other`` (a view of the same type whose rows are ``v_other_stride`` apart) by the weight ``mix`` (float32 [1])
     where it is given.  Heads are ``padded`` values wide in the queries and the pools, zeros at their end."""
@@ -981,9 +982,15 @@ def attention_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off
     t, w = proj.shape
     if max(q_off + heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim, g_off + (heads if gated else 0)) > w:
         raise KernelError("attention_prep: the projection's rows are shorter than q, k, v and the gates")
-    for name, wt in (("q", q_weight), ("k", k_weight)):
-        if wt is not None:
-            _need(wt, f"attention_prep {name} norm weight", dtype=torch.float32, shape=(dim,))
+    q_weight_stride = 0
+    if q_weight is not None and q_weight.ndim == 2:
+        # a weight of its own for every query head
+        _need(q_weight, "attention_prep q norm weights", dtype=torch.float32, shape=(heads, dim))
+        q_weight_stride = dim
+    elif q_weight is not None:
+        _need(q_weight, "attention_prep q norm weight", dtype=torch.float32, shape=(dim,))
+    if k_weight is not None:
+        _need(k_weight, "attention_prep k norm weight", dtype=torch.float32, shape=(dim,))
     if pairs:
         _need(cos_sin, "attention_prep cos/sin", dtype=torch.float32, shape=(t, pairs, 2))
     page_size = pool_slots = 0
@@ -1004,7 +1011,8 @@ def attention_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off
     check(load().fsie_attention_prep(proj.data_ptr(), w, q_off, k_off, v_off, g_off, heads, kv_heads, dim, vdim, padded,
                                      _ptr(q_weight), _ptr(k_weight), float(eps), pairs, _ptr(cos_sin), _ptr(v_other),
                                      int(v_other_stride), _ptr(mix), q.data_ptr(), _ptr(gate), _ptr(slots), _ptr(k_pool),
-                                     _ptr(v_pool), page_size, pool_slots, t, dtype_code(proj.dtype), _stream()))
+                                     _ptr(v_pool), page_size, pool_slots, t, dtype_code(proj.dtype), q_weight_stride,
+                                     _stream()))
     return q, gate
 
 
@@ -1019,4 +1027,177 @@ def gate_heads(x: torch.Tensor, padded: int, vdim: int, heads: int, gate: Option
         _need(gate, "gate_heads gate", dtype=torch.float32, shape=(t, heads))
     y = torch.empty((t, heads * vdim), dtype=x.dtype, device=x.device)
     check(load().fsie_gate_heads(x.data_ptr(), padded, _ptr(gate), y.data_ptr(), t, heads, vdim, dtype_code(x.dtype), _stream()))
+    return y
+
+
+def group_rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, out_dtype: torch.dtype,
+                  delta: Optional[torch.Tensor] = None, delta2: Optional[torch.Tensor] = None, delta_scale: float = 1.0,
+                  weight2: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None, write_back: bool = False):
+    """RMS norm in ``groups`` equal consecutive parts of ``residual + delta_scale * (delta + delta2)`` (float32 stream
+    [T, H]; each delta [T, H] in float32 or bfloat16, or None), every part divided by its own root mean square, times
+    ``weight`` (float32).  ``write_back`` stores the sum into ``residual``; ``rows`` (int32) selects rows.  With
+    ``weight2`` the result is a pair: the same normed rows times either weight."""
+    _need(residual, "group_rmsnorm residual", dtype=torch.float32, ndim=2)
+    t, h = residual.shape
+    _need(weight, "group_rmsnorm weight", dtype=torch.float32, shape=(h,))
+    if weight2 is not None:
+        _need(weight2, "group_rmsnorm second weight", dtype=torch.float32, shape=(h,))
+    for name, d in (("delta", delta), ("delta2", delta2)):
+        if d is not None:
+            _need(d, f"group_rmsnorm {name}", shape=(t, h))
+    n_rows = t
+    if rows is not None:
+        _need(rows, "group_rmsnorm rows", dtype=torch.int32, ndim=1)
+        n_rows = rows.shape[0]
+    out = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device)
+    out2 = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device) if weight2 is not None else None
+    check(load().fsie_group_rmsnorm(residual.data_ptr(), _ptr(delta), dtype_code(delta.dtype) if delta is not None else 0,
+                                    _ptr(delta2), dtype_code(delta2.dtype) if delta2 is not None else 0, float(delta_scale),
+                                    weight.data_ptr(), _ptr(weight2), out.data_ptr(), _ptr(out2), _ptr(rows), n_rows, h,
+                                    int(groups), float(eps), dtype_code(out_dtype), int(write_back), _stream()))
+    return out if weight2 is None else (out, out2)
+
+
+def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, q_starts: torch.Tensor, seq_slots: torch.Tensor,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """``x + conv(x)``: a causal convolution over time within every request, channel by channel.  ``x`` float32 [T, H];
+    ``weight`` float32 [H, taps], the last tap on the token itself; ``state`` float32 [slots, ..., taps - 1, H], a view
+    whose first dimension are the requests' slots: the inputs before a portion's first token (oldest first), brought
+    up to date by this call.  The result has ``out_dtype``."""
+    _need(x, "causal_conv x", dtype=torch.float32, ndim=2)
+    t, h = x.shape
+    _need(weight, "causal_conv weight", dtype=torch.float32, ndim=2)
+    taps = weight.shape[1]
+    if weight.shape[0] != h or taps < 1:
+        raise KernelError(f"causal_conv: weight {tuple(weight.shape)} does not fit rows of {h}")
+    if taps > 1 and (not isinstance(state, torch.Tensor) or not state.is_cuda or state.dtype != torch.float32 or state.ndim != 3
+                     or tuple(state.shape[1:]) != (taps - 1, h) or state.stride(2) != 1 or state.stride(1) != h):
+        raise KernelError(f"causal_conv: the state must be float32 [slots, {taps - 1}, {h}] with contiguous records")
+    _need(q_starts, "causal_conv q_starts", dtype=torch.int32, ndim=1)
+    _need(seq_slots, "causal_conv seq_slots", dtype=torch.int32, ndim=1)
+    y = torch.empty((t, h), dtype=out_dtype, device=x.device)
+    check(load().fsie_causal_conv(x.data_ptr(), weight.data_ptr(), y.data_ptr(), state.data_ptr() if taps > 1 else None,
+                                  state.stride(0) if taps > 1 else 0, state.shape[0] if taps > 1 else 1, q_starts.data_ptr(), seq_slots.data_ptr(), seq_slots.shape[0], t, h, taps,
+                                  dtype_code(out_dtype), _stream()))
+    return y
+
+
+def mlstm_state_floats(dim: int, vdim: int) -> int:
+    """float32 numbers of one head's record of the mLSTM state: S [dim, vdim], n [dim], m and three unused ones."""
+    return int(load().fsie_mlstm_state_floats(dim, vdim))
+
+
+def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: torch.Tensor, gate_cap: float, q_scale: float,
+               state: torch.Tensor, q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int):
+    """The matrix memory over the step's tokens, request by request in order.  ``proj`` [T, W] holds q, k (heads * dim
+    each) and v (heads * vdim) at their column offsets; ``gates`` float32 [T, 2 * heads]: the input gates' logits, then
+    the forget gates'; ``state`` float32 [slots, heads, mlstm_state_floats(dim, vdim)], updated in place.  Returns
+    (num [T, heads, vdim], den [T, heads], coef [T, heads, 4]), all float32: S^T q, n . q and (keep, take, exp(-m), m)."""
+    _need(proj, "mlstm proj", ndim=2)
+    t, w = proj.shape
+    if max(q_off + heads * dim, k_off + heads * dim, v_off + heads * vdim) > w:
+        raise KernelError("mlstm_scan: the projection's rows are shorter than q, k and v")
+    _need(gates, "mlstm gates", dtype=torch.float32, shape=(t, 2 * heads))
+    _need(state, "mlstm state", dtype=torch.float32, ndim=3)
+    if tuple(state.shape[1:]) != (heads, mlstm_state_floats(dim, vdim)):
+        raise KernelError(f"mlstm_scan: state {tuple(state.shape)} is not [slots, {heads}, {mlstm_state_floats(dim, vdim)}]")
+    _need(q_starts, "mlstm q_starts", dtype=torch.int32, ndim=1)
+    _need(seq_slots, "mlstm seq_slots", dtype=torch.int32, ndim=1)
+    num = torch.empty((t, heads, vdim), dtype=torch.float32, device=proj.device)
+    den = torch.empty((t, heads), dtype=torch.float32, device=proj.device)
+    coef = torch.empty((t, heads, 4), dtype=torch.float32, device=proj.device)
+    check(load().fsie_mlstm_scan(proj.data_ptr(), w, q_off, k_off, v_off, dtype_code(proj.dtype), gates.data_ptr(),
+                                 float(gate_cap), float(q_scale), state.data_ptr(), state.shape[0], q_starts.data_ptr(),
+                                 seq_slots.data_ptr(), seq_slots.shape[0], t, heads, dim, vdim, coef.data_ptr(),
+                                 num.data_ptr(), den.data_ptr(), _stream()))
+    return num, den, coef
+
+
+def mlstm_out(num: torch.Tensor, den: torch.Tensor, coef: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float,
+              out_dtype: torch.dtype) -> torch.Tensor:
+    """[T, heads * vdim] in ``out_dtype``: every head's num / (max(|den|, exp(-m)) + 1e-6) divided by its root mean square,
+    times ``weight`` (float32 [heads * vdim]) and the sigmoid of ``gate`` ([T, heads * vdim], a view whose rows may be
+    a stride apart)."""
+    _need(num, "mlstm num", dtype=torch.float32, ndim=3)
+    t, heads, vdim = num.shape
+    _need(den, "mlstm den", dtype=torch.float32, shape=(t, heads))
+    _need(coef, "mlstm coef", dtype=torch.float32, shape=(t, heads, 4))
+    _need(weight, "mlstm norm weight", dtype=torch.float32, shape=(heads * vdim,))
+    if not gate.is_cuda or gate.dtype != out_dtype or tuple(gate.shape) != (t, heads * vdim) or gate.stride(1) != 1:
+        raise KernelError("mlstm_out: the gate must be [T, heads * vdim] of the output's type with contiguous rows")
+    y = torch.empty((t, heads * vdim), dtype=out_dtype, device=num.device)
+    check(load().fsie_mlstm_out(num.data_ptr(), den.data_ptr(), coef.data_ptr(), gate.data_ptr(), gate.stride(0),
+                                weight.data_ptr(), y.data_ptr(), t, heads, vdim, float(eps), dtype_code(out_dtype), _stream()))
+    return y
+
+
+MOE_TILE_ROWS = 16
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int, scale: float):
+    """(ids int32 [T, top], weights float32 [T, top]): the ``top`` experts with the largest sigmoid(x . router^T) +
+    correction (ties: the lower index) and their weights, the chosen sigmoids divided by their sum times ``scale``.
+    ``x`` [T, H] and ``router`` [E, H] share a type; the logits are summed in float32."""
+    _need(x, "moe_route x", ndim=2)
+    t, h = x.shape
+    _need(router, "moe_route router", dtype=x.dtype, ndim=2)
+    e = router.shape[0]
+    if router.shape[1] != h:
+        raise KernelError(f"moe_route: router {tuple(router.shape)} does not fit rows of {h}")
+    _need(correction, "moe_route correction", dtype=torch.float32, shape=(e,))
+    ids = torch.empty((t, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((t, top), dtype=torch.float32, device=x.device)
+    check(load().fsie_moe_route(x.data_ptr(), router.data_ptr(), correction.data_ptr(), dtype_code(x.dtype), ids.data_ptr(),
+                                weights.data_ptr(), t, h, e, int(top), float(scale), _stream()))
+    return ids, weights
+
+
+def moe_group(ids: torch.Tensor, experts: int):
+    """The (token, choice) pairs of ``ids`` [T, top] grouped by expert: (order int32 [pairs]: the pair in every slot,
+    slot_of int32 [pairs], tiles int32 [max_tiles, 3]: (expert, first slot, slots) of every tile of MOE_TILE_ROWS
+    slots; unused tiles have no slots)."""
+    _need(ids, "moe_group ids", dtype=torch.int32, ndim=2)
+    n = ids.numel()
+    max_tiles = -(-n // MOE_TILE_ROWS) + experts
+    order = torch.empty((n,), dtype=torch.int32, device=ids.device)
+    slot_of = torch.empty((n,), dtype=torch.int32, device=ids.device)
+    tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=ids.device)
+    check(load().fsie_moe_group(ids.data_ptr(), n, int(experts), MOE_TILE_ROWS, order.data_ptr(), slot_of.data_ptr(),
+                                tiles.data_ptr(), max_tiles, _stream()))
+    return order, slot_of, tiles
+
+
+def moe_gemm(a: torch.Tensor, weight: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, gather_div: int = 0,
+             pair_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One product per expert: out[slot] = a[row(slot)] . weight[expert of slot]^T with ``weight`` [E, N, K].
+    ``gather_div`` > 0: row(slot) = order[slot] // gather_div (``a`` holds tokens); 0: row(slot) = slot.  Without
+    ``pair_weight`` the result is the exact GELU of the product in ``a``'s type; with it (float32 [pairs]) the product
+    times the pair's weight, float32."""
+    _need(a, "moe_gemm a", ndim=2)
+    _need(weight, "moe_gemm weight", dtype=a.dtype, ndim=3)
+    _, n, k = weight.shape
+    if a.shape[1] != k:
+        raise KernelError(f"moe_gemm: rows of {a.shape[1]} against weights {tuple(weight.shape)}")
+    _need(tiles, "moe_gemm tiles", dtype=torch.int32, ndim=2)
+    _need(order, "moe_gemm order", dtype=torch.int32, ndim=1)
+    slots = order.shape[0]
+    if not gather_div and a.shape[0] != slots:
+        raise KernelError("moe_gemm: without a gather the rows are the slots")
+    if pair_weight is not None:
+        _need(pair_weight, "moe_gemm pair weights", dtype=torch.float32)
+        if pair_weight.numel() != slots:
+            raise KernelError("moe_gemm: one weight a pair")
+    out = torch.empty((slots, n), dtype=torch.float32 if pair_weight is not None else a.dtype, device=a.device)
+    check(load().fsie_moe_gemm(a.data_ptr(), weight.data_ptr(), out.data_ptr(), tiles.data_ptr(), tiles.shape[0],
+                               order.data_ptr(), int(gather_div), _ptr(pair_weight), n, k, 1 if pair_weight is not None else 0,
+                               dtype_code(a.dtype), MOE_TILE_ROWS, _stream()))
+    return out
+
+
+def moe_combine(rows: torch.Tensor, slot_of: torch.Tensor, n_tokens: int, top: int) -> torch.Tensor:
+    """float32 [T, H]: for every token the sum of its ``top`` rows (``rows`` [pairs, H] by slot), in the order of its choices."""
+    _need(rows, "moe_combine rows", dtype=torch.float32, ndim=2)
+    _need(slot_of, "moe_combine slot_of", dtype=torch.int32, shape=(n_tokens * top,))
+    y = torch.empty((n_tokens, rows.shape[1]), dtype=torch.float32, device=rows.device)
+    check(load().fsie_moe_combine(rows.data_ptr(), slot_of.data_ptr(), y.data_ptr(), n_tokens, top, rows.shape[1], _stream()))
     return y

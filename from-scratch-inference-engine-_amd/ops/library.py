@@ -26,7 +26,7 @@ _SIGNATURES = {
     "fsie_version": ([], c_int),
     "fsie_device_info": ([c_char_p, c_int, ctypes.POINTER(c_int)], c_int),
     "fsie_device_compute_units": ([], c_int),
-    "fsie_embedding": ([_P, c_int, _P, _P, c_int, c_int, c_int, _P], c_int),
+    "fsie_embedding": ([_P, c_int, _P, _P, c_int, c_int, c_int, c_float, _P], c_int),
     "fsie_rmsnorm": ([_P, _P, _P, _P, _P, c_int, c_int, c_float, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_rmsnorm_plain": ([_P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_zero_rows": ([_P, _P, c_int, c_int64, c_int, _P], c_int),
@@ -53,16 +53,16 @@ _SIGNATURES = {
     "fsie_fragment_order_size": ([c_int, c_int], c_int64),
     "fsie_fragment_order": ([_P, _P, c_int, c_int, _P], c_int),
     "fsie_attention_scalar": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
-                               c_int, c_int, c_float, c_int, _P, _P], c_int),
+                               c_int, c_int, c_float, c_int, _P, c_float, _P], c_int),
     "fsie_attention_mfma": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
-                             c_int, c_int, c_float, c_int, c_int, _P, _P], c_int),
+                             c_int, c_int, c_float, c_int, c_int, _P, c_float, _P], c_int),
     "fsie_attention_mfma_qkv_ok": ([c_int, c_int], c_int),
     "fsie_attention_mfma_qkv": ([_P, c_int, c_int, _P, _P, _P, _P, _P, c_int64, _P, c_int, _P, c_int, _P, _P, c_int,
                                  c_int, c_int, c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_attention_mfma_max_waves": ([c_int], c_int),
     "fsie_attention_mfma_lds_ok": ([c_int, c_int], c_int),
     "fsie_attention_mfma_lds": ([_P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int,
-                                 c_float, _P, _P], c_int),
+                                 c_float, _P, c_float, _P], c_int),
     "fsie_attention_mfma_tiles": ([c_int, c_int], c_int),
     "fsie_attention_merge": ([_P, _P, c_int, _P, c_int, c_int, c_int, _P, _P], c_int),
     "fsie_attention_scalar_tile_tokens": ([c_int, c_int], c_int),
@@ -90,8 +90,19 @@ _SIGNATURES = {
     "fsie_pair_embedding": ([_P, _P, c_int, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int64, c_int64,
                              c_float, _P], c_int),
     "fsie_attention_prep": ([_P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float,
-                             c_int, _P, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, _P], c_int),
+                             c_int, _P, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, _P], c_int),
     "fsie_gate_heads": ([_P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_group_rmsnorm": ([_P, _P, c_int, _P, c_int, c_float, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int,
+                            _P], c_int),
+    "fsie_causal_conv": ([_P, _P, _P, _P, c_int64, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_mlstm_state_floats": ([c_int, c_int], c_int64),
+    "fsie_mlstm_scan": ([_P, c_int64, c_int, c_int, c_int, c_int, _P, c_float, c_float, _P, c_int, _P, _P, c_int, c_int, c_int,
+                         c_int, c_int, _P, _P, _P, _P], c_int),
+    "fsie_mlstm_out": ([_P, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_float, c_int, _P], c_int),
+    "fsie_moe_route": ([_P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_float, _P], c_int),
+    "fsie_moe_group": ([_P, c_int, c_int, c_int, _P, _P, _P, c_int, _P], c_int),
+    "fsie_moe_gemm": ([_P, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_moe_combine": ([_P, _P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_sample": ([_P, c_int, c_int, _P, _P, _P, _P, _P, _P], c_int),
 }
 

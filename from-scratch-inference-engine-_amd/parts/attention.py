@@ -353,12 +353,15 @@ class AttentionPlanner:
 
 def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n_kv: int, head_dim: int,
                     window: Optional[int], scale: float, n_tokens: int, sinks: Optional[torch.Tensor] = None,
-                    share_keys: bool = True) -> torch.Tensor:
+                    share_keys: bool = True, softcap: Optional[float] = None) -> torch.Tensor:
     """Causal attention of a step's queries over the paged cache, by the work items of ``plan`` (an
     ``AttentionPlanner``'s): [n_tokens, n_heads * head_dim] in the queries' type.  ``q``: rows of ``q_stride``
     values whose first n_heads * head_dim are the heads' queries; the keys and values of the step's own
     tokens are in the cache already.  ``sinks`` (float32 [n_heads] or None): a term exp(sinks[h]) more in the
-    denominator of head h's softmax.  Every mixer whose cache is pages of keys and values calls this."""
+    denominator of head h's softmax.  ``softcap`` (a positive number or None): the scaled scores become
+    softcap * tanh(score / softcap) before the mask and the softmax.  Every mixer whose cache is pages of keys and
+    values calls this."""
+    cap = float(softcap or 0.0)
     out = torch.empty((n_tokens, n_heads * head_dim), dtype=q.dtype, device=q.device)
     partials = None
     if plan.n_partial:
@@ -367,21 +370,21 @@ def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n
     if plan.mfma:
         if plan.n_small:
             ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
-                               plan.n_small, out, *args, large=False, waves=plan.waves, sinks=sinks)
+                               plan.n_small, out, *args, large=False, waves=plan.waves, sinks=sinks, softcap=cap)
         if plan.n_large and not plan.n_long and share_keys and ops.attention_mfma_lds_ok(head_dim, cache.page_size):
             ops.attention_mfma_lds(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
                                    plan.items[plan.n_small:], plan.groups, plan.n_groups, out, n_heads,
-                                   n_kv, head_dim, window, scale, n_tokens, sinks=sinks)
+                                   n_kv, head_dim, window, scale, n_tokens, sinks=sinks, softcap=cap)
         elif plan.n_large:
             ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
-                               plan.items[plan.n_small:], plan.n_large, out, *args, large=True, sinks=sinks)
+                               plan.items[plan.n_small:], plan.n_large, out, *args, large=True, sinks=sinks, softcap=cap)
         if plan.n_long:
             ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
                                plan.items[plan.n_small + plan.n_large:], plan.n_long, out, *args, large=True,
-                               waves=4, sinks=sinks)
+                               waves=4, sinks=sinks, softcap=cap)
     else:
         ops.attention_scalar(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
-                             plan.n_small + plan.n_large, out, *args, sinks=sinks)
+                             plan.n_small + plan.n_large, out, *args, sinks=sinks, softcap=cap)
     if plan.n_merges:
         ops.attention_merge(partials, plan.merges, plan.n_merges, out, n_heads, head_dim, sinks=sinks)
     return out
@@ -402,7 +405,12 @@ class GQAttention(Mixer):
     its row's product with x before the output projection.  ``value_mix``: "source" publishes this layer's
     values of the step's tokens, "mixed" replaces its own by (1 - w) v + w v_source (parameter
     ``value_mix_weight``, one number) before they are cached; both ends must agree in kv heads and value size.
-    With any of the last three, what stands between projection and attention is one kernel
+    ``o_bias=True``: the output projection has a bias.  ``unit_norm_eps``: every q and k head is divided by its root
+    mean square (eps inside the root; no weight; a rotation does not change a head's root mean square, so the kernel's
+    order, norm then rotation, gives the same head as rotation then norm).  ``head_temperature=True`` (with
+    ``unit_norm_eps``): a number per query head (parameter ``temperature``) multiplies its scores.  ``softcap``: the
+    scaled scores become softcap * tanh(score / softcap).
+    With any of gate, mixed values, another value size or the unit norm, what stands between projection and attention is one kernel
     (``ops.attention_prep``: head norms, rotation of the first ``rotary_dim`` values from the step's table, value
     mixing, gates, cache write) and one after it (``ops.gate_heads``).
 
@@ -430,7 +438,9 @@ class GQAttention(Mixer):
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
                  position: PositionEncoding, window: Optional[int] = None, q_norm: Optional[Norm] = None,
                  k_norm: Optional[Norm] = None, sink: bool = False, keep_first: int = 0, scale: Optional[float] = None,
-                 value_dim: Optional[int] = None, gate: bool = False, value_mix: Optional[str] = None):
+                 value_dim: Optional[int] = None, gate: bool = False, value_mix: Optional[str] = None,
+                 o_bias: bool = False, unit_norm_eps: Optional[float] = None, head_temperature: bool = False,
+                 softcap: Optional[float] = None):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: heads {n_heads} must be a multiple of kv heads {n_kv_heads}")
         self.value_dim = head_dim if value_dim is None else int(value_dim)
@@ -447,7 +457,18 @@ class GQAttention(Mixer):
         self.position = position
         self.q_norm, self.k_norm = q_norm, k_norm
         self.has_gate, self.value_mix = bool(gate), value_mix
-        self.prepared = self.has_gate or value_mix is not None or self.value_dim != head_dim
+        self.unit_norm_eps = None if unit_norm_eps is None else float(unit_norm_eps)
+        self.has_temperature = bool(head_temperature)
+        if self.unit_norm_eps is not None and (q_norm is not None or k_norm is not None):
+            raise ValueError("attention: the heads take norm parts or the unit norm, not both")
+        if self.has_temperature and self.unit_norm_eps is None:
+            raise ValueError("attention: a temperature a head goes with the unit norm of the heads")
+        if softcap is not None and not softcap > 0:
+            raise ValueError(f"attention: softcap {softcap} must be positive")
+        self.softcap = None if softcap is None else float(softcap)
+        self.temperature: Optional[torch.Tensor] = None
+        self._unit_q = self._unit_k = None  # the unit norm's weights: the temperature (or 1) for q, 1 for k
+        self.prepared = self.has_gate or value_mix is not None or self.value_dim != head_dim or self.unit_norm_eps is not None
         if self.prepared:
             if position.rotates and getattr(position, "layout", None) != "half":
                 raise ValueError("attention: with a gate, mixed values or values of another size the position encoding "
@@ -457,7 +478,7 @@ class GQAttention(Mixer):
         self.rot_pairs = (getattr(position, "rotary_dim", 0) // 2) if position.rotates else 0
         self.q_dim, self.kv_dim, self.v_dim = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * self.value_dim
         self.qkv = Linear(hidden_size, self.q_dim + self.kv_dim + self.v_dim + (n_heads if gate else 0), bias=qkv_bias)
-        self.o = Linear(n_heads * self.value_dim, hidden_size)
+        self.o = Linear(n_heads * self.value_dim, hidden_size, bias=o_bias)
         self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
         self._planner: Optional[AttentionPlanner] = None
         self.has_sink = bool(sink)
@@ -478,7 +499,12 @@ class GQAttention(Mixer):
         decls = {"qkv_weight": ParamDecl((rows, self.hidden_size)),
                  "o_weight": ParamDecl((self.hidden_size, self.n_heads * self.value_dim))}
         if self.qkv.has_bias:
-            decls["qkv_bias"] = ParamDecl((rows,), "vector", "bias")
+            # (the gates' rows have no bias in a checkpoint: theirs is zero, added in ``prepare``)
+            decls["qkv_bias"] = ParamDecl((rows - (self.n_heads if self.has_gate else 0),), "vector", "bias")
+        if self.o.has_bias:
+            decls["o_bias"] = ParamDecl((self.hidden_size,), "vector", "bias")
+        if self.has_temperature:
+            decls["temperature"] = ParamDecl((self.n_heads,), "vector", "norm")
         if self.has_sink:
             decls["sink"] = ParamDecl((self.n_heads,), "vector", "bias")
         if self.value_mix is not None:
@@ -489,8 +515,16 @@ class GQAttention(Mixer):
     qkv_weight = property(lambda s: s.qkv.weight, lambda s, t: setattr(s.qkv, "weight", t))
     qkv_bias = property(lambda s: s.qkv.bias, lambda s, t: setattr(s.qkv, "bias", t))
     o_weight = property(lambda s: s.o.weight, lambda s, t: setattr(s.o, "weight", t))
+    o_bias = property(lambda s: s.o.bias, lambda s, t: setattr(s.o, "bias", t))
 
     def prepare(self, device, compute_dtype) -> None:
+        bias = self.qkv.bias
+        if self.has_gate and bias is not None and bias.shape[0] == self.qkv.out_features - self.n_heads:
+            self.qkv.bias = torch.cat([bias, torch.zeros((self.n_heads,), dtype=bias.dtype, device=bias.device)])
+        if self.unit_norm_eps is not None:
+            ones = torch.ones((self.n_heads, self.head_dim), dtype=torch.float32, device=device)
+            self._unit_k = ones[0].contiguous()
+            self._unit_q = ones if self.temperature is None else (ones * self.temperature.to(device)[:, None]).contiguous()
         copies = bool(self.options.get("weight_copies", True))
         self.o.prepare(copies)
         self.qkv.prepare(copies)  # (read by the product of 17 to 64 rows; the few-rows product with the rotation reads rows)
@@ -519,7 +553,7 @@ class GQAttention(Mixer):
     def _from_sums(self, x: torch.Tensor, ctx, cache, plan, table) -> Optional[torch.Tensor]:
         """Attention of a step of one token a request straight from the q/k/v product's partial sums
         (None: not such a step, or the kernels do not take the sizes)."""
-        if not (self.finish_qkv_in_attention and self.sink is None and not self.keep_first and table is not None and cache.writes and plan.mfma and plan.single
+        if not (self.finish_qkv_in_attention and self.sink is None and not self.keep_first and self.softcap is None and table is not None and cache.writes and plan.mfma and plan.single
                 and plan.n_small and not plan.n_large and not plan.n_long and x.dtype == torch.bfloat16
                 and ops.attention_mfma_qkv_ok(self.head_dim, cache.page_size)):
             return None
@@ -596,15 +630,18 @@ class GQAttention(Mixer):
                 raise RuntimeError("attention: no earlier layer of this step has published values to mix with")
             other_stride = other.stride(0)
         norm = self.q_norm if self.q_norm is not None else self.k_norm
+        q_weight = None if self.q_norm is None else self.q_norm.weight
+        k_weight = None if self.k_norm is None else self.k_norm.weight
+        eps = norm.eps if norm is not None else 0.0
+        if self.unit_norm_eps is not None:
+            q_weight, k_weight, eps = self._unit_q, self._unit_k, self.unit_norm_eps
         store = dict(slots=cache.slots, k_pool=cache.k_pool, v_pool=cache.v_pool) if cache.writes else {}
-        q, gate = ops.attention_prep(proj, 0, k_off, v_off, g_off, nh, nkv, hd, vd, pd,
-                                     None if self.q_norm is None else self.q_norm.weight,
-                                     None if self.k_norm is None else self.k_norm.weight,
-                                     norm.eps if norm is not None else 0.0, self.rot_pairs, table, self.has_gate,
+        q, gate = ops.attention_prep(proj, 0, k_off, v_off, g_off, nh, nkv, hd, vd, pd, q_weight, k_weight, eps,
+                                     self.rot_pairs, table, self.has_gate,
                                      v_other=other, v_other_stride=other_stride,
                                      mix=self.value_mix_weight if other is not None else None, **store)
         out = paged_attention(q, nh * pd, cache, plan, nh, nkv, pd, self.window, self.scale, x.shape[0], sinks=self.sink,
-                              share_keys=self.share_keys)
+                              share_keys=self.share_keys, softcap=self.softcap)
         if gate is not None or pd != vd:
             out = ops.gate_heads(out, pd, vd, nh, gate)
         return self.o.for_residual(out, ctx)
@@ -619,5 +656,5 @@ class GQAttention(Mixer):
             return self.o.for_residual(out, ctx)
         qkv = self._project_rotate_store(x, ctx, cache, table)
         out = paged_attention(qkv, qkv.shape[1], cache, plan, self.n_heads, self.n_kv, self.head_dim, self.window,
-                              self.scale, x.shape[0], sinks=self.sink, share_keys=self.share_keys)
+                              self.scale, x.shape[0], sinks=self.sink, share_keys=self.share_keys, softcap=self.softcap)
         return self.o.for_residual(out, ctx)

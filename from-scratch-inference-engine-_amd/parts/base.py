@@ -50,15 +50,17 @@ class HiddenState:
     pending delta goes through before it is added (a layer that also norms its sublayers' outputs), or
     None; the norm that folds the delta in applies it in the same pass.  ``delta2``: a second pending delta of
     the same kinds, left by a block whose mixer and feed-forward read the same stream (only norms that set
-    ``adds_two_deltas`` take it; the others refuse)."""
+    ``adds_two_deltas`` take it; the others refuse).  ``delta_scale``: a factor on the pending deltas when they are
+    added, x += delta_scale * (delta + delta2) (only norms that set ``scales_deltas`` take another value than 1)."""
 
-    __slots__ = ("residual", "delta", "delta_norm", "delta2")
+    __slots__ = ("residual", "delta", "delta_norm", "delta2", "delta_scale")
 
     def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None, delta_norm=None):
         self.residual = residual
         self.delta = delta
         self.delta_norm = delta_norm
         self.delta2 = None
+        self.delta_scale = 1.0
 
 
 class Part:
@@ -114,6 +116,8 @@ class Norm(Part):
     # True if the norm adds a second pending delta (``HiddenState.delta2``) in the same pass, and offers
     # ``pair(hidden, other, out_dtype)``: this norm's and another one's output of the same stream at once
     adds_two_deltas = False
+    # True if the norm multiplies the pending deltas by ``HiddenState.delta_scale`` as it adds them
+    scales_deltas = False
 
     def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
         raise NotImplementedError
@@ -170,16 +174,36 @@ class PositionEncoding(Part):
         return None
 
 
+class Convolution(Part):
+    """A short causal convolution over time in front of a sublayer: ``y = conv.forward(x, ctx, state)`` with ``x``
+    float32 [T, H]; ``state_shape()`` is what it keeps per request (the inputs that the next portion still needs)
+    and ``state`` the view [slots, *state_shape] of the block's per-request memory that belongs to it."""
+
+    kind = "convolution"
+
+    def state_shape(self) -> Tuple[int, ...]:
+        raise NotImplementedError
+
+    def forward(self, x: torch.Tensor, ctx, state: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Block(Part):
     kind = "block"
 
-    def forward(self, hidden: HiddenState, ctx, cache) -> None:
+    def state_need(self):
+        """What the block itself keeps for a request between steps, beside its mixer's cache: a per-request need of
+        ``cache.needs`` (a ``StateNeed``), or None.  The model allocates it and hands ``forward`` its view as
+        ``state`` (a ``LayerCache`` whose ``state`` is [slots + 1, *shape], indexed by ``ctx.seq_slots``)."""
+        return None
+
+    def forward(self, hidden: HiddenState, ctx, cache, state=None) -> None:
         raise NotImplementedError
 
 
 # ------------------------------------------------------------------------------ registries
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Part]]] = {
-    "norm": {}, "mixer": {}, "feed_forward": {}, "position": {}, "block": {},
+    "norm": {}, "mixer": {}, "feed_forward": {}, "position": {}, "block": {}, "convolution": {},
 }
 
 

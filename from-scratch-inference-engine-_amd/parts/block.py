@@ -4,7 +4,9 @@ from __future__ import annotations
 
 from typing import Dict, Optional
 
-from .base import Block, FeedForward, HiddenState, Mixer, Norm, Part, register_part
+import torch
+
+from .base import Block, Convolution, FeedForward, HiddenState, Mixer, Norm, Part, register_part
 
 
 @register_part("block", "pre_norm")
@@ -63,27 +65,72 @@ class ParallelBlock(Block):
     """Mixer and feed-forward side by side: x += mixer(norm1(x)) + ffn(norm2(x)), both norms of the same x.  The two
     outputs stay pending in the hidden state as two deltas, and the norm that reads the stream next adds both in
     the pass that normalises; this block's two norms are one pass as well (``Norm.pair``).  ``ffn=None``: the layer
-    has no feed-forward (and no second norm)."""
+    has no feed-forward (and no second norm).  ``residual_scale`` = m: x += m * (mixer(..) + ffn(..)); the factor
+    travels with the pending deltas (norms that set ``scales_deltas``).  ``mixer_conv`` / ``ffn_conv``: a short causal
+    convolution between a norm and its sublayer; what they keep per request is the block's own state."""
 
     graph_safe = True
 
-    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None):
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None,
+                 residual_scale: float = 1.0, mixer_conv: Optional[Convolution] = None,
+                 ffn_conv: Optional[Convolution] = None):
         if (ffn is None) != (ffn_norm is None):
             raise ValueError("parallel block: a feed-forward comes with its norm, or neither")
+        if ffn is None and ffn_conv is not None:
+            raise ValueError("parallel block: a convolution in front of a feed-forward that is not there")
         if not mixer_norm.adds_two_deltas or (ffn_norm is not None and not ffn_norm.adds_two_deltas):
             raise ValueError("parallel block: its norms must add two pending deltas and come as a pair (layer_norm does)")
+        self.residual_scale = float(residual_scale)
+        if self.residual_scale != 1.0 and not (mixer_norm.scales_deltas and (ffn_norm is None or ffn_norm.scales_deltas)):
+            raise ValueError("parallel block: a factor on the sublayers' sum needs norms that apply it (group_rms_norm does)")
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+        self.mixer_conv, self.ffn_conv = mixer_conv, ffn_conv
+        self._convs = [c for c in (mixer_conv, ffn_conv) if c is not None]
+        if len({c.state_shape() for c in self._convs}) > 1:
+            raise ValueError("parallel block: its convolutions must keep states of one shape")
 
     def sub_parts(self) -> Dict[str, Part]:
         parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
         if self.ffn is not None:
             parts.update(ffn_norm=self.ffn_norm, ffn=self.ffn)
+        if self.mixer_conv is not None:
+            parts["mixer_conv"] = self.mixer_conv
+        if self.ffn_conv is not None:
+            parts["ffn_conv"] = self.ffn_conv
         return parts
 
-    def forward(self, hidden: HiddenState, ctx, cache) -> None:
+    def state_need(self):
+        if not self._convs or 0 in self._convs[0].state_shape():
+            return None  # (a convolution of one tap keeps nothing)
+        from ..cache.needs import StateNeed
+
+        return StateNeed((len(self._convs), *self._convs[0].state_shape()), "float32")
+
+    def _conv(self, conv: Optional[Convolution], x: torch.Tensor, ctx, state) -> torch.Tensor:
+        if conv is None:
+            return x
+        if 0 in conv.state_shape():
+            return conv.forward(x, ctx, None)
+        if state is None or state.state is None:
+            raise RuntimeError("parallel block: no state for its convolutions (the model did not ask for the block's need)")
+        return conv.forward(x, ctx, state.state[:, self._convs.index(conv)])
+
+    def forward(self, hidden: HiddenState, ctx, cache, state=None) -> None:
+        # a convolution reads the norm's output before any rounding and rounds once itself
+        a_type = torch.float32 if self.mixer_conv is not None else ctx.compute_dtype
         if self.ffn is None:
-            hidden.delta = self.mixer.forward(self.mixer_norm(hidden, ctx.compute_dtype), ctx, cache)
+            a = self._conv(self.mixer_conv, self.mixer_norm(hidden, a_type), ctx, state)
+            hidden.delta = self.mixer.forward(a, ctx, cache)
+            hidden.delta_scale = self.residual_scale
             return
-        a, b = self.mixer_norm.pair(hidden, self.ffn_norm, ctx.compute_dtype)
+        b_type = torch.float32 if self.ffn_conv is not None else ctx.compute_dtype
+        if a_type == b_type:
+            a, b = self.mixer_norm.pair(hidden, self.ffn_norm, a_type)
+        else:
+            a = self.mixer_norm(hidden, a_type)  # (adds the pending deltas; the second norm then finds none)
+            b = self.ffn_norm(hidden, b_type)
+        a = self._conv(self.mixer_conv, a, ctx, state)
+        b = self._conv(self.ffn_conv, b, ctx, state)
         hidden.delta = self.mixer.forward(a, ctx, cache)
         hidden.delta2 = self.ffn.forward(b, ctx)
+        hidden.delta_scale = self.residual_scale

@@ -12,21 +12,22 @@ from .linear import Linear
 
 
 class TokenEmbedding(Part):
-    """x[t] = table[ids[t]] without scaling (src/model/nn.cpp:90-108), written as the float32
-    residual stream."""
+    """x[t] = table[ids[t]] (src/model/nn.cpp:90-108, which does not scale) times ``scale``, written as
+    the float32 residual stream."""
 
     kind = "embedding"
     graph_safe = True  # reads the step's token ids from the device
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0):
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.scale = float(scale)
         self.weight = None
 
     def param_decls(self) -> Dict[str, ParamDecl]:
         return {"weight": ParamDecl((self.vocab_size, self.hidden_size))}
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return ops.embedding(self.weight, ids)
+        return ops.embedding(self.weight, ids, scale=self.scale)
 
     def cache_need(self):
         """What the embedding keeps for a request between steps (a need of ``cache.needs``), or None."""
@@ -47,7 +48,7 @@ class PairHashEmbedding(TokenEmbedding):
     graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int, mul_cur: int, scale: float = 1.0):
-        super().__init__(vocab_size, hidden_size)
+        super().__init__(vocab_size, hidden_size, scale)
         if buckets < 1:
             raise ValueError(f"pair embedding: buckets {buckets} must be positive")
         self.buckets, self.mul_prev, self.mul_cur, self.scale = int(buckets), int(mul_prev), int(mul_cur), float(scale)

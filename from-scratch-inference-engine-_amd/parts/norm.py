@@ -11,6 +11,9 @@ from .base import HiddenState, Norm, ParamDecl, register_part
 
 
 def _no_second_delta(hidden: HiddenState, name: str) -> None:
+    if hidden.delta_scale != 1.0:
+        raise RuntimeError(f"{name}: the stream's pending delta carries a factor of {hidden.delta_scale}, which this norm "
+                           f"does not apply")
     if hidden.delta2 is not None:
         raise RuntimeError(f"{name}: the stream has a second pending delta (a block whose sublayers read the same "
                            f"stream came before), which this norm does not add")
@@ -92,6 +95,8 @@ class LayerNorm(Norm):
     def _take(hidden: HiddenState, clear: bool):
         if hidden.delta_norm is not None:
             raise RuntimeError("layer_norm: a pending delta with a norm of its own is not taken")
+        if hidden.delta_scale != 1.0:
+            raise RuntimeError("layer_norm: a factor on the pending deltas is not applied")
         deltas = hidden.delta, hidden.delta2
         if clear:
             hidden.delta = hidden.delta2 = None
@@ -112,3 +117,58 @@ class LayerNorm(Norm):
     def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         d1, d2 = self._take(hidden, False)
         return ops.layer_norm(hidden.residual, self.weight, self.bias, self.eps, out_dtype, delta=d1, delta2=d2, rows=rows)
+
+
+@register_part("norm", "group_rms_norm")
+class GroupRMSNorm(Norm):
+    """RMS norm in groups: the row is cut into ``groups`` equal consecutive parts, each divided by its own
+    sqrt(mean(part^2) + eps), and the whole multiplied by w; everything in float32.  The row is
+    x = residual + delta_scale * (delta + delta2): up to two pending deltas (each in the compute type or float32)
+    and the stream's factor on them, added in the pass that normalises.  ``pair`` gives this norm's and another
+    one's output of the same stream from one pass (they differ in the weight only).  ``groups=1`` is the plain RMS
+    norm with those additions."""
+
+    adds_partial_sums = False  # (a delta cut into partial sums is not taken: the model then never makes one)
+    adds_two_deltas = True
+    scales_deltas = True
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, eps: float, groups: int = 1):
+        if groups < 1 or hidden_size % groups:
+            raise ValueError(f"group_rms_norm: {hidden_size} values do not make {groups} equal groups")
+        self.hidden_size, self.eps, self.groups = hidden_size, float(eps), int(groups)
+        self.weight = None
+
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        return {"weight": ParamDecl((self.hidden_size,), "vector", "norm")}
+
+    @staticmethod
+    def _take(hidden: HiddenState, clear: bool):
+        if hidden.delta_norm is not None:
+            raise RuntimeError("group_rms_norm: a pending delta with a norm of its own is not taken")
+        taken = hidden.delta, hidden.delta2, hidden.delta_scale
+        for d in taken[:2]:
+            if d is not None and d.ndim != 2:
+                raise RuntimeError("group_rms_norm: a pending delta of partial sums is not taken")
+        if clear:
+            hidden.delta = hidden.delta2 = None
+            hidden.delta_scale = 1.0
+        return taken
+
+    def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
+        d1, d2, scale = self._take(hidden, True)
+        return ops.group_rmsnorm(hidden.residual, self.weight, self.eps, self.groups, out_dtype, delta=d1, delta2=d2,
+                                 delta_scale=scale, write_back=d1 is not None or d2 is not None)
+
+    def pair(self, hidden: HiddenState, other: "GroupRMSNorm", out_dtype: torch.dtype):
+        if (not isinstance(other, GroupRMSNorm) or other.eps != self.eps or other.hidden_size != self.hidden_size
+                or other.groups != self.groups):
+            raise ValueError("group_rms_norm: a pair is two such norms of one width, eps and number of groups")
+        d1, d2, scale = self._take(hidden, True)
+        return ops.group_rmsnorm(hidden.residual, self.weight, self.eps, self.groups, out_dtype, delta=d1, delta2=d2,
+                                 delta_scale=scale, weight2=other.weight, write_back=d1 is not None or d2 is not None)
+
+    def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        d1, d2, scale = self._take(hidden, False)
+        return ops.group_rmsnorm(hidden.residual, self.weight, self.eps, self.groups, out_dtype, delta=d1, delta2=d2,
+                                 delta_scale=scale, rows=rows)
