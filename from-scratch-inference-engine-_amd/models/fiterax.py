@@ -85,8 +85,8 @@ def build_fiterax(cfg: FiteraxConfig) -> ModelSpec:
     final_norm = norm("final.norm")
     lm_head = LMHead(w, cfg.vocab)
     bind(bindings, lm_head, "weight", [TensorSpec("head", (cfg.vocab, w))])
-    # a layer without feed-forward may still carry the tensors of a convolution in front of one: not read
-    unused = tuple(f"l{i}.canon2" for i, layer in enumerate(cfg.layers) if layer.mlp is None)
+    # a layer without feed-forward may still carry the norm and the convolution in front of one: not read
+    unused = tuple(f"l{i}.{name}" for i, layer in enumerate(cfg.layers) if layer.mlp is None for name in ("norm2", "canon2"))
     return ModelSpec(config=cfg, embedding=embedding, layers=layers, schedule=schedule, final_norm=final_norm,
                      lm_head=lm_head, bindings=bindings, ignore_unexpected=unused)
 
