@@ -97,6 +97,24 @@ def rotate_half(x, positions, base, dims):
     return out
 
 
+def capped_attention(q, k, v, scale, temps, cap, past=0):
+    """q [n, heads, dim] at positions past .. past + n - 1 against k [total, kv, dim], v [total, kv, vdim]: scores times
+    ``scale`` and the head's temperature, capped (cap * tanh(score / cap); None: not), causal softmax.  [n, heads, vdim]."""
+    n, heads, _ = q.shape
+    total, kv, vdim = v.shape
+    out = np.zeros((n, heads, vdim))
+    seen = np.arange(total)[None, :] <= (past + np.arange(n))[:, None]
+    for hd in range(heads):
+        g = hd // (heads // kv)
+        s = (q[:, hd] @ k[:, g].T) * scale * (1.0 if temps is None else temps[hd])
+        if cap:
+            s = cap * np.tanh(s / cap)
+        s = np.where(seen, s, -np.inf)
+        e = np.exp(s - s.max(-1, keepdims=True))
+        out[:, hd] = (e / e.sum(-1, keepdims=True)) @ v[:, g]
+    return out
+
+
 def attention_mixer(h, w, p, m, eps):
     """Grouped-query attention with biases, partly rotated and unit-normed q and k, a temperature a head, capped
     scores, and a sigmoid gate a head on the result."""
@@ -110,33 +128,19 @@ def attention_mixer(h, w, p, m, eps):
     q = unit_rms(rotate_half(q, pos, rot.get("base", 1.0), rot.get("dims", 0)), eps)
     k = unit_rms(rotate_half(k, pos, rot.get("base", 1.0), rot.get("dims", 0)), eps)
     gate = sigmoid(h @ w[p + "g"].T)  # [T, heads]
-    cap = m.get("softcap")
-    out = np.zeros((t, heads, vdim))
-    causal = np.tril(np.ones((t, t), dtype=bool))
-    for hd in range(heads):
-        g = hd // (heads // kv)
-        s = (q[:, hd] @ k[:, g].T) * m["scale"] * w[p + "temp"][hd]
-        if cap:
-            s = cap * np.tanh(s / cap)
-        s = np.where(causal, s, -np.inf)
-        s = s - s.max(-1, keepdims=True)
-        e = np.exp(s)
-        out[:, hd] = (e / e.sum(-1, keepdims=True)) @ v[:, g]
+    out = capped_attention(q, k, v, m["scale"], w[p + "temp"], m.get("softcap"))
     out = out * gate[:, :, None]
     return out.reshape(t, heads * vdim) @ w[p + "o"].T + w[p + "o.b"]
 
 
-def mlstm_mixer(h, w, p, m, eps):
-    """Matrix memory with exponential gates: per head S [dim, vdim], n [dim] and a running maximum m that starts
-    at zero; token by token."""
-    t = h.shape[0]
-    heads, dim, vdim, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
-    q = (h @ w[p + "q"].T).reshape(t, heads, dim) * dim ** -0.5
-    k = (h @ w[p + "k"].T).reshape(t, heads, dim)
-    v = (h @ w[p + "v"].T).reshape(t, heads, vdim)
-    gi = cap * np.tanh((h @ w[p + "i"].T + w[p + "i.b"]) / cap)
-    gf = log_sigmoid(cap * np.tanh((h @ w[p + "f"].T + w[p + "f.b"]) / cap))
+def matrix_memory(q, k, v, gi, gf, pieces=False):
+    """q, k [T, heads, dim], v [T, heads, vdim], log input gates gi and log forget gates gf [T, heads]: per head
+    S [dim, vdim], n [dim] and a running maximum that all start at zero; token by token.  [T, heads, vdim].
+    ``pieces``: also what the quotient is made of, (S^T q [T, heads, vdim], n . q [T, heads], the maximum [T, heads])."""
+    t, heads, dim = q.shape
+    vdim = v.shape[2]
     out = np.zeros((t, heads, vdim))
+    num, den, top = np.zeros((t, heads, vdim)), np.zeros((t, heads)), np.zeros((t, heads))
     for hd in range(heads):
         S, n, mx = np.zeros((dim, vdim)), np.zeros(dim), 0.0
         for i in range(t):
@@ -145,7 +149,24 @@ def mlstm_mixer(h, w, p, m, eps):
             S = keep * S + take * np.outer(k[i, hd], v[i, hd])
             n = keep * n + take * k[i, hd]
             mx = new
-            out[i, hd] = (S.T @ q[i, hd]) / (max(abs(n @ q[i, hd]), math.exp(-mx)) + 1e-6)
+            num[i, hd], den[i, hd], top[i, hd] = S.T @ q[i, hd], n @ q[i, hd], mx
+            out[i, hd] = num[i, hd] / (max(abs(den[i, hd]), math.exp(-mx)) + 1e-6)
+    return (out, num, den, top) if pieces else out
+
+
+def capped_gates(zi, zf, cap):
+    """(log input gate, log forget gate) from the gates' logits."""
+    return cap * np.tanh(zi / cap), log_sigmoid(cap * np.tanh(zf / cap))
+
+
+def mlstm_mixer(h, w, p, m, eps):
+    t = h.shape[0]
+    heads, dim, vdim = m["heads"], m["dim"], m["vdim"]
+    q = (h @ w[p + "q"].T).reshape(t, heads, dim) * dim ** -0.5
+    k = (h @ w[p + "k"].T).reshape(t, heads, dim)
+    v = (h @ w[p + "v"].T).reshape(t, heads, vdim)
+    gi, gf = capped_gates(h @ w[p + "i"].T + w[p + "i.b"], h @ w[p + "f"].T + w[p + "f.b"], m["gate_cap"])
+    out = matrix_memory(q, k, v, gi, gf)
     out = unit_rms(out, eps).reshape(t, heads * vdim) * w[p + "norm"]
     out = out * sigmoid(h @ w[p + "g"].T)
     return out @ w[p + "o"].T
