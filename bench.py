@@ -269,12 +269,27 @@ def botulorn_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
             "layers": out}
 
 
-DESIGN_SHAPES = {"gilozen": gilozen_shape, "botulorn": botulorn_shape}
+def fiterax_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Fiterax configuration of real layer sizes: an mLSTM matrix memory and grouped-query attention in turn (capped
+    scores, unit-normed heads, 64 rotated values), every layer with eight routed experts beside its mixer, two a token;
+    the experts together hold as many weights as the dense feed-forward of the same ``ff``."""
+    heads = width // 128
+    memory = {"heads": width // 256, "dim": 128, "vdim": 256, "gate_cap": 15.0}
+    gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
+           "rot": {"base": 500000.0, "dims": 64}}
+    mlp = {"kind": "moe", "expert": {"ff": ff * 3 // 16}, "router": {"experts": 8, "top": 2, "scale": 2.5}}
+    out = [{"type": "mlstm" if i % 2 == 0 else "attention", "mixer": dict(memory if i % 2 == 0 else gqa), "mlp": dict(mlp)}
+           for i in range(layers)]
+    return {"architecture": "Fiterax", "width": width, "vocab": vocab, "norm": {"eps": 1e-5, "groups": 2},
+            "embedding": {"scale": 12.0}, "residual_mult": 0.3, "canon": {"taps": 4}, "layers": out}
+
+
+DESIGN_SHAPES = {"gilozen": gilozen_shape, "botulorn": botulorn_shape, "fiterax": fiterax_shape}
 DESIGN_SIZES = {"2048": (2048, 8192, 9, 32000), "4096": (4096, 14336, 9, 32000)}  # width, ff, layers, vocab
 
 
 def design_comparison(args) -> int:
-    """--workload gilozen | botulorn: prefill (one prompt of 2,048 tokens in one step) and decode (batches of 8 and 64 at a
+    """--workload gilozen | botulorn | fiterax: prefill (one prompt of 2,048 tokens in one step) and decode (batches of 8 and 64 at a
     context of 512, from captured graphs) of the named design at two real layer sizes with random weights, beside a Qwen2
     model of the same width, feed-forward, layers and vocabulary (grouped-query attention, 128 values a head, four
     query heads a key/value head) through the same step function.  One JSON line."""
@@ -359,14 +374,14 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
     ap.add_argument("--no-streamed-copies", action="store_true",
                     help="do not keep the large weights a second time in the order of the matrix instruction's fragments")
-    ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen | botulorn: widths to run (2048, 4096)")
-    ap.add_argument("--design-batches", default="8,64", help="--workload gilozen | botulorn: decode batches to time (at most 64)")
-    ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen | botulorn: what to time (for a trace of one phase)")
-    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen", "botulorn"], default="decode",
+    ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen | botulorn | fiterax: widths to run (2048, 4096)")
+    ap.add_argument("--design-batches", default="8,64", help="--workload gilozen | botulorn | fiterax: decode batches to time (at most 64)")
+    ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen | botulorn | fiterax: what to time (for a trace of one phase)")
+    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen", "botulorn", "fiterax"], default="decode",
                     help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "
                          "--outputs tokens each, through the scheduler (made for --shape 14b).  "
                          "long-prefill: one prompt of --prefill-tokens tokens in portions of the token budget "
-                         "(made for --shape 32b).  gilozen, botulorn: that design beside Qwen2 at equal layer sizes")
+                         "(made for --shape 32b).  gilozen, botulorn, fiterax: that design beside Qwen2 at equal layer sizes")
     ap.add_argument("--requests", type=int, default=32)
     ap.add_argument("--min-prompt", type=int, default=128)
     ap.add_argument("--max-prompt", type=int, default=4096)
