@@ -263,7 +263,7 @@ int fsie_causal_conv(const float* x, const float* w, void* y, float* state, int6
 // ---- mLSTM: a matrix memory with exponential gates ------------------------------------------------
 // gates [n_tokens][2 * heads] float32 (input gate logits, then forget gate logits); per request and head the running
 // maximum m (state record's last part) is carried: i = cap tanh(gi / cap), f = logsigmoid(cap tanh(gf / cap)),
-// m_t = max(f + m_(t-1), i).  Writes coef [n_tokens][heads][4] = (exp(f + m_(t-1) - m_t), exp(i - m_t), exp(-m_t), m_t).
+// m_t = max(f + m_(t-1), i).  Writes coef [n_tokens][heads][4] = (f, i, m_(t-1), m_t).
 // Then the memory: S_t = keep S_(t-1) + take k v^T, n_t likewise with k alone; num[t][h][:] = S_t^T q, den[t][h] = n_t . q
 // (q scaled by q_scale).  proj [n_tokens][stride] holds q (heads * dim from q_off), k (from k_off), v (heads * vdim
 // from v_off).  state [n_slots][heads][dim * vdim + dim + 4] float32: S, n, m (and three unused numbers).
@@ -271,7 +271,10 @@ int64_t fsie_mlstm_state_floats(int dim, int vdim);
 int fsie_mlstm_scan(const void* proj, int64_t stride, int q_off, int k_off, int v_off, int dtype, const float* gates,
                     float gate_cap, float q_scale, float* state, int n_slots, const int32_t* q_starts,
                     const int32_t* seq_slots, int n_seqs, int n_tokens, int heads, int dim, int vdim, float* coef,
-                    float* num, float* den, hipStream_t stream);
+                    float* num, float* den, float* chunk_work, int max_chunks, hipStream_t stream);
+// The chunk kernels' work array: with `chunk_work` (room for max_chunks >= n_tokens / chunk_tokens + n_seqs chunks of
+// chunk_floats floats) the portions of at least chunk_min tokens go sixteen tokens at a time on the matrix cores.
+int fsie_mlstm_scan_shape(int heads, int dim, int vdim, int* chunk_tokens, int* chunk_min, int64_t* chunk_floats);
 // y[t][h][:] = unit_rms(num / (max(|den|, exp(-m)) + 1e-6)) * weight[h][:] * sigmoid(gate[t][h][:]), y in `dtype`;
 // gate rows lie `gate_stride` values apart (columns of the fused projection)
 int fsie_mlstm_out(const float* num, const float* den, const float* coef, const void* gate, int64_t gate_stride,

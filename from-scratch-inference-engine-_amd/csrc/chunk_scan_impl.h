@@ -41,12 +41,16 @@ __host__ __device__ inline int64_t gla_chunk_floats(int dp) { return static_cast
 // A wave's chain per chunk is nine matrix instructions; the waves' shares of the chunks' o (and the four steps
 // of A v, dealt to the waves in turn) meet in shared memory, a barrier every few chunks, and are added in the
 // order of the waves.  The shares of o that the token-by-token kernel would leave in further planes of `out` are zero here.
-template <typename T, int NW>
+//
+// ONES: the grid has one more tile of columns after the head's last, and that tile carries a single further column
+// of S whose values v are all one: a normaliser n_t = diag(g) n_(t-1) + k_t, with o = q . n.  It lies at
+// `ones_at` floats into the head's record, its channels side by side, and its o goes to ones_out [tokens][heads].
+template <typename T, int NW, bool ONES>
 __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int v_off, const float* __restrict__ work,
     float* __restrict__ state, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots,
     float* __restrict__ out, int64_t out_plane, int heads, int dim, int vdim, int dp, int planes, int n_slots,
-    int64_t state_head_stride) {
+    int64_t state_head_stride, int64_t ones_at, float* __restrict__ ones_out) {
     constexpr int G = NW <= 8 ? 4 : 2;  // chunks between two barriers: their shares of o lie in LDS side by side
     __shared__ float part[2][G][NW][4][64];
     const int seq = blockIdx.x, h = blockIdx.y;
@@ -58,17 +62,19 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, g4 = lane >> 4;
+    const bool ones_tile = ONES && blockIdx.z == gridDim.z - 1;  // the same for the whole workgroup
     const int col = blockIdx.z * 16 + n;
-    const bool col_ok = col < vdim;
+    const bool col_ok = ones_tile ? n == 0 : col < vdim;
+    const int64_t row_stride = ones_tile ? 1 : vdim;
     const int ch0 = wave * 16;  // this wave's first key channel
 
     // (a head's S [dim][vdim] starts every state_head_stride floats: the mixer may keep more than S in a head's record)
-    float* my_state = state + (static_cast<int64_t>(slot) * heads + h) * state_head_stride + col;
+    float* my_state = state + (static_cast<int64_t>(slot) * heads + h) * state_head_stride + (ones_tile ? ones_at : col);
     floatx4 S;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = ch0 + 4 * g4 + i;
-        S[i] = (col_ok && row < dim) ? my_state[static_cast<int64_t>(row) * vdim] : 0.f;
+        S[i] = (col_ok && row < dim) ? my_state[static_cast<int64_t>(row) * row_stride] : 0.f;
     }
     const int64_t per_chunk = gla_chunk_floats(dp) * heads;
     const float* w = work + (static_cast<int64_t>(first) * heads + h) * gla_chunk_floats(dp);
@@ -96,7 +102,10 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
         const T* vc = vp + static_cast<int64_t>(t0) * proj_stride;
         // (a token past the portion's end has q = k = 0 and a zero row and column of A: the v of the portion's
         // last token stands in for it, a number that is multiplied by zero)
-        if (t0 + kGlaChunk <= hi) {  // the same in all lanes
+        if (ones_tile) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) v[slot_][m] = 1.f;
+        } else if (t0 + kGlaChunk <= hi) {  // the same in all lanes
 #pragma unroll
             for (int m = 0; m < 4; ++m) v[slot_][m] = to_float(vc[v_at[m]]);
         } else {
@@ -114,7 +123,9 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
     // order of the waves, a value a thread and round.  Further planes of `out`: zeros.
     auto finish = [&](int gi, int count, bool really) {
         const int t0 = lo + gi * G * kGlaChunk;
-        float* oc = out + static_cast<int64_t>(t0) * out_stride + h * vdim + blockIdx.z * 16;
+        float* oc = ones_tile ? ones_out + static_cast<int64_t>(t0) * heads + h
+                              : out + static_cast<int64_t>(t0) * out_stride + h * vdim + blockIdx.z * 16;
+        const int o_stride = ones_tile ? heads : static_cast<int>(out_stride);
 #pragma unroll
         for (int e0 = 0; e0 < 256 * G; e0 += 64 * NW) {
             const int e = e0 + tid;
@@ -124,10 +135,11 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
 #pragma unroll
                 for (int ww = 1; ww < NW; ++ww) sum += part[gi & 1][j][ww][i][l];
                 const int tok = j * kGlaChunk + 4 * (l >> 4) + i, c = l & 15;
-                if (really && t0 + tok < hi && blockIdx.z * 16 + c < vdim) {
-                    float* dst = oc + tok * static_cast<int>(out_stride) + c;
+                if (really && t0 + tok < hi && (ones_tile ? c == 0 : blockIdx.z * 16 + c < vdim)) {
+                    float* dst = oc + tok * o_stride + c;
                     *dst = sum;
-                    for (int pl = 1; pl < planes; ++pl) dst[pl * out_plane] = 0.f;
+                    if (!ones_tile)
+                        for (int pl = 1; pl < planes; ++pl) dst[pl * out_plane] = 0.f;
                 }
             }
         }
@@ -172,7 +184,7 @@ __global__ __launch_bounds__(64 * NW) void gla_chunk_scan_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = ch0 + 4 * g4 + i;
-        if (col_ok && row < dim) my_state[static_cast<int64_t>(row) * vdim] = S[i];
+        if (col_ok && row < dim) my_state[static_cast<int64_t>(row) * row_stride] = S[i];
     }
 }
 

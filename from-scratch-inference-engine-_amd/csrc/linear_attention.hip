@@ -326,10 +326,10 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     int scan_waves = 1;  // a wave for every sixteen key channels, rounded up to a power of two: at most sixteen
     while (scan_waves * 16 < dim) scan_waves *= 2;
 #define FSIE_GLA_CHUNKS(T, NW)                                                                                        \
-    gla_chunk_scan_kernel<T, NW><<<scan_grid, 64 * NW, 0, stream>>>(static_cast<const T*>(proj), proj_stride, v_off,    \
+    gla_chunk_scan_kernel<T, NW, false><<<scan_grid, 64 * NW, 0, stream>>>(static_cast<const T*>(proj), proj_stride, v_off,    \
                                                                     chunk_work, state, q_starts, seq_slots, out,        \
                                                                     out_plane, heads, dim, vdim, dp, splits, n_slots,           \
-                                                                    static_cast<int64_t>(dim) * vdim)
+                                                                    static_cast<int64_t>(dim) * vdim, 0, nullptr)
 #define FSIE_GLA_LAUNCH(T, ROWS)                                                                                       \
     gla_scan_kernel<T, ROWS><<<grid, kGlaThreads, 0, stream>>>(static_cast<const T*>(proj), proj_stride, v_off, prep, plane, \
                                                                state, q_starts, seq_slots, out, out_plane, heads, dim, vdim, \

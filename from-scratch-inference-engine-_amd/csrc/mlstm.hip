@@ -7,55 +7,174 @@
 //   o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
 //
 // S, n and m start at zero and live in the request's state record [heads][dim * vdim + dim + 4] (float32).  Both
-// exponents are never positive.  Three kernels a step:
-//   gates  one thread a (request, head): the activations of all its tokens, then the running maximum in order; it
-//          carries m in the state and leaves (keep, take, exp(-m), m) per token and head
-//   scan   a wave per (request, head, 16 value columns) walks the request's tokens in order; lane = (channel
-//          quarter, column) holds a quarter of the key channels of its column of S in registers and the four quarters'
-//          shares of S^T q meet through lane exchanges; one more wave per (request, head) carries n and leaves n . q
+// exponents are never positive.  The kernels of a step:
+//   gates  a wave per (request, head): the activations of 64 tokens at a time, a token a lane, then the running
+//          maximum in the tokens' order (the same few instructions in all lanes); it carries m in the state and
+//          leaves (f, i, m before, m) per token and head
+//   scan   portions below sixteen tokens, single decoded tokens among them: a wave per (request, head, 16 value
+//          columns) walks the tokens in order; lane = (channel quarter, column) holds a quarter of the key channels of
+//          its column of S in registers and the four quarters' shares of S^T q meet through lane exchanges; one more
+//          wave per (request, head) carries n and leaves n . q
+//   chunks longer portions go sixteen tokens at a time on the matrix cores.  With b_t the sum of f over the chunk's
+//          tokens up to t and m_in the maximum that the chunk starts from,
+//            S_t = exp(b_t + m_in - m_t) S_in + sum_{j <= t} exp(b_t - b_j + i_j - m_t) k_j v_j^T,
+//          which is the recurrence with its factors multiplied out; m_t is at least every exponent's positive part, so
+//          none is positive here either.  A first kernel lays out, per chunk and head, q_t exp(b_t + m_in - m_t),
+//          k_j exp(b_last - b_j + i_j - m_last), the chunk's decay exp(b_last + m_in - m_last) and
+//          A[t][j] = (q_t . k_j) exp(b_t - b_j + i_j - m_t); the walk over chunks that the recurrent mixers share
+//          does the rest, with n as one more column of S whose values are all one.
 //   out    a wave per (token, head): the division, the head's unit RMS, the weight and the sigmoid gate
-// Everything here is float32 whatever the projections' type.  The numbers of a token do not depend on how the
-// request's tokens were cut into steps: the walk is token by token in both cases.
+// Everything here is float32 whatever the projections' type.  Which way a portion goes depends on its own length
+// alone, and the two ways differ by rounding only.
 #include "common.h"
 #include "api.h"
+#include "chunk_scan_impl.h"
 
 namespace {
 
 constexpr int kCols = 16;        // value columns a wave
 constexpr int kQuarters = 4;     // lane groups that split the key channels
 constexpr int kMaxDim = 512;     // key channels a head
+constexpr int kMaxChunkDim = 256;  // ... of a head whose long portions go chunk by chunk
+constexpr int kPrepThreads = 256;
 
 __device__ __forceinline__ float log_sigmoid(float z) {
     // -log(1 + exp(-z)), without overflow at either end
     return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
 }
 
-__global__ void mlstm_gates_kernel(const float* __restrict__ gates, float cap, float* __restrict__ state, int64_t record,
-                                   int64_t m_at, int n_slots, const int32_t* __restrict__ q_starts,
-                                   const int32_t* __restrict__ seq_slots, int n_seqs, int heads, float* __restrict__ coef) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= n_seqs * heads) return;
-    const int s = idx / heads, h = idx - s * heads;
+// grid = requests * heads waves
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(const float* __restrict__ gates, float cap, float* __restrict__ state,
+                                                         int64_t record, int64_t m_at, int n_slots,
+                                                         const int32_t* __restrict__ q_starts,
+                                                         const int32_t* __restrict__ seq_slots, int heads,
+                                                         float* __restrict__ coef) {
+    const int s = blockIdx.x / heads, h = blockIdx.x - s * heads;
+    const int lane = threadIdx.x;
     const int slot = seq_slots[s];
     const int first = q_starts[s], last = q_starts[s + 1];
+    if (last <= first) return;
     float* m_state = (slot >= 0 && slot < n_slots) ? state + (static_cast<int64_t>(slot) * heads + h) * record + m_at : nullptr;
     float m = m_state ? *m_state : 0.f;
-    for (int t = first; t < last; ++t) {
-        const float gi = gates[static_cast<int64_t>(t) * 2 * heads + h];
-        const float gf = gates[static_cast<int64_t>(t) * 2 * heads + heads + h];
-        const float i = cap * tanhf(gi / cap);
-        const float f = log_sigmoid(cap * tanhf(gf / cap));
-        const float carried = f + m;
-        const float m_new = fmaxf(carried, i);
-        float4 c;
-        c.x = expf(carried - m_new);
-        c.y = expf(i - m_new);
-        c.z = expf(-m_new);
-        c.w = m_new;
-        *reinterpret_cast<float4*>(coef + (static_cast<int64_t>(t) * heads + h) * 4) = c;
-        m = m_new;
+    for (int t0 = first; t0 < last; t0 += 64) {
+        const int t = t0 + lane;
+        const int nt = min(64, last - t0);  // the same in all lanes
+        float f = 0.f, i = 0.f;
+        if (t < last) {
+            const float gi = gates[static_cast<int64_t>(t) * 2 * heads + h];
+            const float gf = gates[static_cast<int64_t>(t) * 2 * heads + heads + h];
+            i = cap * tanhf(gi / cap);
+            f = log_sigmoid(cap * tanhf(gf / cap));
+        }
+        float before = 0.f, mine = 0.f;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            if (j < nt) {
+                const float fj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f), j));
+                const float ij = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, i), j));
+                const float m_new = fmaxf(fj + m, ij);
+                if (lane == j) before = m, mine = m_new;
+                m = m_new;
+            }
+        }
+        if (t < last) *reinterpret_cast<float4*>(coef + (static_cast<int64_t>(t) * heads + h) * 4) = float4{f, i, before, mine};
     }
-    if (m_state && last > first) *m_state = m;
+    if (m_state && lane == 0) *m_state = m;
+}
+
+// grid = (upper bound of the step's chunks, heads); the chunks of a step are numbered request by request.  Work array
+// of a chunk and head as the walk over chunks wants it: qd [16][dp], kdT [dp][16], g [dp], A [16][16].
+template <typename T>
+__global__ __launch_bounds__(kPrepThreads) void mlstm_chunk_prep_kernel(
+    const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off, const float* __restrict__ coef,
+    float* __restrict__ work, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots, int n_seqs,
+    int heads, int dim, int dp, float q_scale, int n_slots) {
+    extern __shared__ float lds[];  // [2][16][dp + 4]: q, k
+    __shared__ float s_dq[kGlaChunk], s_dk[kGlaChunk], s_b[kGlaChunk], s_i[kGlaChunk], s_m[kGlaChunk], s_g;
+    const int ld = dp + 4;
+    float* qs = lds;
+    float* ks = qs + kGlaChunk * ld;
+    const int h = blockIdx.y, tid = threadIdx.x;
+    int first = 0, seq = -1;
+    for (int s = 0; s < n_seqs; ++s) {
+        const int n = gla_chunks_of(q_starts, seq_slots, s, n_slots);
+        if (static_cast<int>(blockIdx.x) < first + n) { seq = s; break; }
+        first += n;
+    }
+    if (seq < 0) return;  // the same for the whole workgroup
+    const int t0 = q_starts[seq] + (static_cast<int>(blockIdx.x) - first) * kGlaChunk;
+    const int nt = min(kGlaChunk, q_starts[seq + 1] - t0);
+    float* w = work + (static_cast<int64_t>(blockIdx.x) * heads + h) * gla_chunk_floats(dp);
+    float* qd = w;
+    float* kdT = qd + kGlaChunk * dp;
+    float* g = kdT + kGlaChunk * dp;
+    float* A = g + dp;
+
+    if (tid < kGlaChunk) {
+        // b_t, in the tokens' order; the tokens past the portion's end stand still (f = 0, k = q = 0)
+        const float4* cf = reinterpret_cast<const float4*>(coef) + static_cast<int64_t>(t0) * heads + h;
+        const float m_in = cf[0].z;
+        float b = 0.f, b_mine = 0.f, b_last = 0.f;
+        for (int j = 0; j < nt; ++j) {
+            b += cf[static_cast<int64_t>(j) * heads].x;
+            if (j == tid) b_mine = b;
+        }
+        b_last = b;
+        const float m_last = cf[static_cast<int64_t>(nt - 1) * heads].w;
+        float dq = 0.f, dk = 0.f, i_mine = 0.f, m_mine = 0.f;
+        if (tid < nt) {
+            const float4 c = cf[static_cast<int64_t>(tid) * heads];
+            dq = expf((b_mine + m_in) - c.w);
+            dk = expf((b_last - b_mine) + (c.y - m_last));
+            i_mine = c.y, m_mine = c.w;
+        }
+        s_dq[tid] = dq, s_dk[tid] = dk, s_b[tid] = b_mine, s_i[tid] = i_mine, s_m[tid] = m_mine;
+        if (tid == 0) s_g = expf(b_last + m_in - m_last);
+    }
+    for (int e = tid; e < kGlaChunk * dp; e += kPrepThreads) {
+        const int t = e / dp, c = e - t * dp;
+        float q = 0.f, k = 0.f;
+        if (t < nt && c < dim) {
+            const T* row = proj + static_cast<int64_t>(t0 + t) * proj_stride + h * dim + c;
+            q = to_float(row[q_off]) * q_scale;
+            k = to_float(row[k_off]);
+        }
+        qs[t * ld + c] = q;
+        ks[t * ld + c] = k;
+    }
+    __syncthreads();
+    for (int e = tid; e < kGlaChunk * dp; e += kPrepThreads) {
+        const int t = e / dp, c = e - t * dp;
+        qd[e] = qs[t * ld + c] * s_dq[t];
+    }
+    for (int e = tid; e < dp * (kGlaChunk / 4); e += kPrepThreads) {
+        const int c = e >> 2, t4 = (e & 3) * 4;
+        floatx4 kd;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kd[i] = ks[(t4 + i) * ld + c] * s_dk[t4 + i];
+        *reinterpret_cast<floatx4*>(kdT + c * kGlaChunk + t4) = kd;
+    }
+    for (int c = tid; c < dp; c += kPrepThreads) g[c] = s_g;
+    // A: thread p < 136 has the pair number p of the rows (r, 15 - r) put side by side, r = p / 17
+    if (tid < kGlaChunk * (kGlaChunk + 1) / 2) {
+        const int r = tid / (kGlaChunk + 1), o = tid - r * (kGlaChunk + 1);
+        const int i = o <= r ? r : kGlaChunk - 1 - r;
+        const int j = o <= r ? o : o - r - 1;
+        float a = 0.f;
+        if (i < nt) {
+            const float* qi = qs + i * ld;
+            const float* kj = ks + j * ld;
+            floatx4 a4 = {0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < dp; c += 4)  // (channels past dim: q = k = 0)
+                a4 += *reinterpret_cast<const floatx4*>(qi + c) * *reinterpret_cast<const floatx4*>(kj + c);
+            a = ((a4[0] + a4[1]) + (a4[2] + a4[3])) * expf((s_b[i] - s_b[j]) + (s_i[j] - s_m[i]));
+        }
+        A[i * kGlaChunk + j] = a;
+    }
+    // above the diagonal: zeros
+    for (int e = tid; e < kGlaChunk * kGlaChunk; e += kPrepThreads) {
+        if ((e & 15) > (e >> 4)) A[e] = 0.f;
+    }
 }
 
 // NI: channels a lane holds (its quarter's share, rounded up); channel of register i: i * 4 + quarter
@@ -65,13 +184,14 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ pr
                                                         int n_slots, const int32_t* __restrict__ q_starts,
                                                         const int32_t* __restrict__ seq_slots, int heads, int dim, int vdim,
                                                         const float* __restrict__ coef, float* __restrict__ num,
-                                                        float* __restrict__ den, int col_tiles) {
+                                                        float* __restrict__ den, int col_tiles, int skip_from) {
     const int s = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
     const int lane = threadIdx.x;
     const int slot = seq_slots[s];
     const int first = q_starts[s], last = q_starts[s + 1];
     if (last <= first) return;
     float* rec = (slot >= 0 && slot < n_slots) ? state + (static_cast<int64_t>(slot) * heads + h) * record : nullptr;
+    if (rec && last - first >= skip_from) return;  // the chunk kernels' portion
     if (tile == col_tiles) {
         // the normaliser: lane l holds channels l, l + 64, ...
         constexpr int NN = (NI * kQuarters + 63) / 64;
@@ -84,7 +204,8 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ pr
         }
         for (int t = first; t < last; ++t) {
             const T* row = proj + static_cast<int64_t>(t) * stride;
-            const float4 cf = *reinterpret_cast<const float4*>(coef + (static_cast<int64_t>(t) * heads + h) * 4);
+            const float4 gm = *reinterpret_cast<const float4*>(coef + (static_cast<int64_t>(t) * heads + h) * 4);
+            const float2 cf = {expf(gm.x + gm.z - gm.w), expf(gm.y - gm.w)};  // keep, take
             float dot = 0.f;
 #pragma unroll
             for (int i = 0; i < NN; ++i) {
@@ -117,7 +238,8 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ pr
     }
     for (int t = first; t < last; ++t) {
         const T* row = proj + static_cast<int64_t>(t) * stride;
-        const float4 cf = *reinterpret_cast<const float4*>(coef + (static_cast<int64_t>(t) * heads + h) * 4);
+        const float4 gm = *reinterpret_cast<const float4*>(coef + (static_cast<int64_t>(t) * heads + h) * 4);
+            const float2 cf = {expf(gm.x + gm.z - gm.w), expf(gm.y - gm.w)};  // keep, take
         const float v = col_in ? to_float(row[v_off + h * vdim + col]) * cf.y : 0.f;  // take * v
         float o = 0.f;
 #pragma unroll
@@ -153,7 +275,7 @@ __global__ __launch_bounds__(256) void mlstm_out_kernel(const float* __restrict_
     const int lane = threadIdx.x & 63;
     const int64_t t = unit / heads;
     const int h = static_cast<int>(unit - t * heads);
-    const float d = 1.0f / (fmaxf(fabsf(den[unit]), coef[unit * 4 + 2]) + 1e-6f);
+    const float d = 1.0f / (fmaxf(fabsf(den[unit]), expf(-coef[unit * 4 + 3])) + 1e-6f);
     const float* o = num + unit * vdim;
     float sum = 0.f;
     for (int j = lane; j < vdim; j += 64) {
@@ -175,10 +297,27 @@ extern "C" int64_t fsie_mlstm_state_floats(int dim, int vdim) {
     return static_cast<int64_t>(dim) * vdim + dim + 4;
 }
 
+// Sizes of the chunk kernels' work array for a layer of these sizes: the tokens of a chunk, the shortest portion that
+// goes chunk by chunk, and the floats of `chunk_work` a chunk (0: heads this wide are walked token by token only).  A
+// step of n_tokens tokens in n_seqs requests has at most n_tokens / chunk_tokens + n_seqs chunks.
+extern "C" int fsie_mlstm_scan_shape(int heads, int dim, int vdim, int* chunk_tokens, int* chunk_min, int64_t* chunk_floats) {
+    FSIE_REQUIRE(heads > 0 && dim > 0 && dim <= kMaxDim && vdim > 0, "mlstm_scan_shape: bad sizes");
+    int waves = 1;
+    while (waves * 16 < dim) waves *= 2;
+    *chunk_tokens = kGlaChunk;
+    *chunk_min = kGlaChunkMin;
+    *chunk_floats = dim <= kMaxChunkDim ? gla_chunk_floats(16 * waves) * heads : 0;
+    return 0;
+}
+
+// chunk_work: room for max_chunks chunks, or null: with it, the portions of at least chunk_min tokens go chunk by
+// chunk (max_chunks must be the bound that fsie_mlstm_scan_shape names, or more); without it every portion is walked
+// token by token.  coef [n_tokens][heads][4] receives (f, i, m before the token, m).
 extern "C" int fsie_mlstm_scan(const void* proj, int64_t stride, int q_off, int k_off, int v_off, int dtype,
                                const float* gates, float gate_cap, float q_scale, float* state, int n_slots,
                                const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, int heads,
-                               int dim, int vdim, float* coef, float* num, float* den, hipStream_t stream) {
+                               int dim, int vdim, float* coef, float* num, float* den, float* chunk_work, int max_chunks,
+                               hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && heads > 0 && dim > 0 && dim <= kMaxDim && vdim > 0 && n_slots > 0,
                  "mlstm_scan: bad sizes T=%d requests=%d heads=%d dim=%d (at most %d) vdim=%d", n_tokens, n_seqs, heads, dim,
                  kMaxDim, vdim);
@@ -186,28 +325,63 @@ extern "C" int fsie_mlstm_scan(const void* proj, int64_t stride, int q_off, int 
     FSIE_REQUIRE(gate_cap > 0.f, "mlstm_scan: the gates' cap must be positive");
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "mlstm_scan: unknown dtype %d", dtype);
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(coef) % 16 == 0, "mlstm_scan: the coefficients must be 16-byte aligned");
+    FSIE_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + heads * dim <= stride && k_off + heads * dim <= stride &&
+                     v_off + heads * vdim <= stride,
+                 "mlstm_scan: the q, k and v columns do not fit a row of %lld", static_cast<long long>(stride));
     if (n_tokens == 0 || n_seqs == 0) return 0;
     const int64_t record = fsie_mlstm_state_floats(dim, vdim);
-    const int64_t m_at = static_cast<int64_t>(dim) * vdim + dim;
-    const int units = n_seqs * heads;
-    mlstm_gates_kernel<<<(units + 63) / 64, 64, 0, stream>>>(gates, gate_cap, state, record, m_at, n_slots, q_starts, seq_slots,
-                                                             n_seqs, heads, coef);
-    FSIE_CHECK_LAUNCH("mlstm_gates");
+    const int64_t n_at = static_cast<int64_t>(dim) * vdim;
+    const int64_t m_at = n_at + dim;
     const int col_tiles = (vdim + kCols - 1) / kCols;
+    FSIE_REQUIRE(heads <= 65535 && col_tiles + 1 <= 65535, "mlstm_scan: too many heads or columns");
+    const bool chunks = chunk_work != nullptr && n_tokens >= kGlaChunkMin && dim <= kMaxChunkDim;
+    if (chunks) {
+        FSIE_REQUIRE(max_chunks >= n_tokens / kGlaChunk + n_seqs, "mlstm_scan: room for %d chunks, the step may have %d",
+                     max_chunks, n_tokens / kGlaChunk + n_seqs);
+        FSIE_REQUIRE(max_chunks <= 0x7fffffff / kGlaChunk, "mlstm_scan: too many chunks");
+        FSIE_REQUIRE(stride <= 0x7fffffff / kGlaChunk && static_cast<int64_t>(heads) * vdim <= 0x7fffffff / kGlaChunk,
+                     "mlstm_scan: rows too long for the chunk kernels' 32-bit offsets");
+        FSIE_REQUIRE(reinterpret_cast<uintptr_t>(chunk_work) % 16 == 0, "mlstm_scan: the work array must be 16-byte aligned");
+    }
+    const int skip_from = chunks ? kGlaChunkMin : 0x7fffffff;
+    mlstm_gates_kernel<<<n_seqs * heads, 64, 0, stream>>>(gates, gate_cap, state, record, m_at, n_slots, q_starts, seq_slots,
+                                                          heads, coef);
+    FSIE_CHECK_LAUNCH("mlstm_gates");
     const dim3 grid(n_seqs, heads, col_tiles + 1);
     const int per_lane = (dim + kQuarters - 1) / kQuarters;
+    int scan_waves = 1;  // a wave for every sixteen key channels, rounded up to a power of two: at most sixteen
+    while (scan_waves * 16 < dim) scan_waves *= 2;
+    const int dp = 16 * scan_waves;
+    const dim3 prep_grid(chunks ? max_chunks : 1, heads);
+    const size_t prep_lds = 2 * kGlaChunk * (dp + 4) * sizeof(float);
+    const int64_t out_plane = static_cast<int64_t>(n_tokens) * heads * vdim;
 #define FSIE_MLSTM(T, NI)                                                                                              \
     mlstm_scan_kernel<T, NI><<<grid, 64, 0, stream>>>(static_cast<const T*>(proj), stride, q_off, k_off, v_off, q_scale, state, \
                                                       record, n_slots, q_starts, seq_slots, heads, dim, vdim, coef, num, den, \
-                                                      col_tiles)
-#define FSIE_MLSTM_T(T)                         \
-    if (per_lane <= 8) FSIE_MLSTM(T, 8);        \
-    else if (per_lane <= 16) FSIE_MLSTM(T, 16); \
-    else if (per_lane <= 32) FSIE_MLSTM(T, 32); \
-    else if (per_lane <= 64) FSIE_MLSTM(T, 64); \
-    else FSIE_MLSTM(T, 128)
+                                                      col_tiles, skip_from)
+#define FSIE_MLSTM_CHUNKS(T, NW)                                                                                       \
+    gla_chunk_scan_kernel<T, NW, true><<<grid, 64 * NW, 0, stream>>>(static_cast<const T*>(proj), stride, v_off, chunk_work,    \
+                                                                     state, q_starts, seq_slots, num, out_plane, heads, dim,   \
+                                                                     vdim, dp, 1, n_slots, record, n_at, den)
+#define FSIE_MLSTM_T(T)                                                                                                \
+    if (per_lane <= 8) FSIE_MLSTM(T, 8);                                                                               \
+    else if (per_lane <= 16) FSIE_MLSTM(T, 16);                                                                        \
+    else if (per_lane <= 32) FSIE_MLSTM(T, 32);                                                                        \
+    else if (per_lane <= 64) FSIE_MLSTM(T, 64);                                                                        \
+    else FSIE_MLSTM(T, 128);                                                                                           \
+    if (chunks) {                                                                                                      \
+        mlstm_chunk_prep_kernel<T><<<prep_grid, kPrepThreads, prep_lds, stream>>>(                                      \
+            static_cast<const T*>(proj), stride, q_off, k_off, coef, chunk_work, q_starts, seq_slots, n_seqs, heads, dim, dp,   \
+            q_scale, n_slots);                                                                                         \
+        if (scan_waves == 1) FSIE_MLSTM_CHUNKS(T, 1);                                                                  \
+        else if (scan_waves == 2) FSIE_MLSTM_CHUNKS(T, 2);                                                             \
+        else if (scan_waves == 4) FSIE_MLSTM_CHUNKS(T, 4);                                                             \
+        else if (scan_waves == 8) FSIE_MLSTM_CHUNKS(T, 8);                                                             \
+        else FSIE_MLSTM_CHUNKS(T, 16);                                                                                 \
+    }
     if (dtype == FSIE_F32) { FSIE_MLSTM_T(float); } else { FSIE_MLSTM_T(bf16_t); }
 #undef FSIE_MLSTM_T
+#undef FSIE_MLSTM_CHUNKS
 #undef FSIE_MLSTM
     FSIE_CHECK_LAUNCH("mlstm_scan");
     return 0;

@@ -5,7 +5,7 @@
 //            score + correction (ties to the lower index), weights = chosen scores / their sum * scale
 //   group    one workgroup: counts per expert, starts, a slot for every pair (pairs of one expert keep the order
 //            of the pairs), and the table of row tiles (expert, first slot, slots) that never cross an expert
-//   gemm     a wave per 16 slots x 64 outputs of one expert's matrix on the matrix cores: bfloat16 operands
+//   gemm     a workgroup per tile of 16, 64 or 128 slots of one expert on the matrix cores: bfloat16 operands
 //            (mfma 16x16x32) or true float32 ones (mfma 16x16x4); both operands run along K in memory, which is
 //            the order the instruction wants; rows are gathered through the order table; the epilogue is the exact
 //            GELU (up) or the pair's routing weight (down, float32 result)
@@ -19,27 +19,62 @@ namespace {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kTileRows = 16;
 constexpr int kMaxExperts = 256;
 constexpr int kMaxTop = 16;
+
+// The logits of kRouteGroup experts at a time: a lane takes 16 bytes of the token's row and of every expert's row
+// per round (all of a round's loads are asked for before any is used), sums its share in the order of the rounds,
+// and the lanes' shares meet in the wave's fixed order.  Rows that are not a whole number of 16 bytes, or not
+// aligned, are read value by value, with the same sums a lane.
+constexpr int kRouteGroup = 8;
 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router,
                                                         const float* __restrict__ correction, int32_t* __restrict__ ids,
                                                         float* __restrict__ weights, int n_tokens, int hidden, int experts,
                                                         int top, float scale) {
+    constexpr int V = 16 / sizeof(T);
     __shared__ float s_score[4][kMaxExperts];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + wave;
     const bool live = t < n_tokens;
     const T* row = x + static_cast<int64_t>(live ? t : 0) * hidden;
     float* score = s_score[wave];
-    for (int e = 0; e < experts && live; ++e) {
-        const T* w = router + static_cast<int64_t>(e) * hidden;
-        float z = 0.f;
-        for (int j = lane; j < hidden; j += 64) z = fmaf(to_float(row[j]), to_float(w[j]), z);
-        z = wave_sum(z);
-        if (lane == 0) score[e] = 1.0f / (1.0f + expf(-z));
+    const bool vec = hidden % V == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(router) & 15) == 0;
+    for (int e0 = 0; e0 < experts && live; e0 += kRouteGroup) {
+        float z[kRouteGroup];
+#pragma unroll
+        for (int i = 0; i < kRouteGroup; ++i) z[i] = 0.f;
+        for (int j = lane * V; j < hidden; j += 64 * V) {
+            union { uint4 raw; T v[V]; } xv, wv[kRouteGroup];
+            if (vec) {
+                xv.raw = *reinterpret_cast<const uint4*>(row + j);
+#pragma unroll
+                for (int i = 0; i < kRouteGroup; ++i) {
+                    const int e = min(e0 + i, experts - 1);  // (past the last: the last once more, dropped below)
+                    wv[i].raw = *reinterpret_cast<const uint4*>(router + static_cast<int64_t>(e) * hidden + j);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < V; ++u) xv.v[u] = j + u < hidden ? row[j + u] : from_float<T>(0.f);
+#pragma unroll
+                for (int i = 0; i < kRouteGroup; ++i) {
+                    const int e = min(e0 + i, experts - 1);
+#pragma unroll
+                    for (int u = 0; u < V; ++u)
+                        wv[i].v[u] = j + u < hidden ? router[static_cast<int64_t>(e) * hidden + j + u] : from_float<T>(0.f);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kRouteGroup; ++i)
+#pragma unroll
+                for (int u = 0; u < V; ++u) z[i] = fmaf(to_float(xv.v[u]), to_float(wv[i].v[u]), z[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < kRouteGroup; ++i) {
+            const float sum = wave_sum(z[i]);
+            if (lane == 0 && e0 + i < experts) score[e0 + i] = 1.0f / (1.0f + expf(-sum));
+        }
     }
     __syncthreads();
     if (!live) return;
@@ -151,87 +186,146 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restri
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
-// A wave: 16 slots x 64 outputs (four 16 x 16 accumulators that share the rows' fragments).  Lane l supplies, for
-// the rows' operand, row l % 16 and the values of K that its lane group (l / 16) owns, and the same of a weight row
-// for the other operand; accumulator register r of lane l is (row 4 (l / 16) + r, column l % 16).
-template <typename T>
+// A workgroup of four waves and a tile of 16 MT slots of one expert.  A wave has MT x NB accumulators of 16 x 16 that
+// share the rows' and the weights' fragments: lane l supplies, for the rows' operand, row l % 16 of each of its MT
+// blocks and the values of K that its lane group (l / 16) owns, and the same of NB weight rows for the other operand;
+// accumulator register r of lane l is (row 4 (l / 16) + r, column l % 16).
+//   KSPLIT false (many rows an expert): the waves take 16 NB outputs each, side by side, and all of K.
+//   KSPLIT true (few rows an expert: the product is bound by the read of the weights): the waves share 16 NB outputs
+//   and take every fourth step of K each; their shares meet in LDS and are added in the order of the waves.
+// A slot's sums depend on the variant, never on the other slots of its tile.
+template <typename T, int MT, int NB, bool KSPLIT>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, const T* __restrict__ w, void* __restrict__ out,
                                                        const int32_t* __restrict__ tiles, const int32_t* __restrict__ order,
                                                        int gather_div, const float* __restrict__ pair_weight, int N, int K,
                                                        int epilogue) {
+    __shared__ float red[KSPLIT ? 3 * MT * NB * 4 * 64 : 1];
     const int32_t* tl = tiles + 3 * blockIdx.x;
     const int expert = tl[0], slot0 = tl[1], n_rows = tl[2];
     if (n_rows <= 0) return;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int n0 = (blockIdx.y * 4 + wave) * 64;
-    if (n0 >= N) return;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int n0 = (KSPLIT ? blockIdx.y : blockIdx.y * 4 + wave) * 16 * NB;
+    if (n0 >= N) return;  // (KSPLIT: the same for the whole workgroup)
     const int r = lane & 15, g = lane >> 4;
-    const bool row_in = r < n_rows;
-    int64_t src = slot0 + r;
-    if (row_in && gather_div > 0) src = order[slot0 + r] / gather_div;
-    const T* arow = a + (row_in ? src : 0) * K;
-    const T* wbase = w + static_cast<int64_t>(expert) * N * K;
-    const T* wrow[4];
-    bool col_in[4];
+    const T* arow[MT];
+    bool row_in[MT];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int i = 0; i < MT; ++i) {
+        row_in[i] = 16 * i + r < n_rows;
+        int64_t src = slot0 + 16 * i + r;
+        if (row_in[i] && gather_div > 0) src = order[src] / gather_div;
+        arow[i] = a + (row_in[i] ? src : 0) * K;
+    }
+    const T* wbase = w + static_cast<int64_t>(expert) * N * K;
+    const T* wrow[NB];
+    bool col_in[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
         const int n = n0 + 16 * j + r;
         col_in[j] = n < N;
         wrow[j] = wbase + static_cast<int64_t>(col_in[j] ? n : 0) * K;
     }
-    floatx4 acc[4];
+    floatx4 acc[MT][NB];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
     if constexpr (sizeof(T) == 2) {
         const bool vec = (K & 7) == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
-        for (int k0 = 0; k0 < K; k0 += 32) {
-            const int k = k0 + 8 * g;
-            union { uint4 raw; bf16x8 v; uint16_t h[8]; } fa, fb[4];
-            fa.raw = uint4{0, 0, 0, 0};
-            if (vec) {
-                if (row_in && k < K) fa.raw = *reinterpret_cast<const uint4*>(arow + k);
+        union Frag { uint4 raw; bf16x8 v; uint16_t h[8]; };
+        if (vec) {
+#pragma unroll 2
+            for (int k0 = KSPLIT ? wave * 32 : 0; k0 < K; k0 += KSPLIT ? 128 : 32) {
+                const int k = k0 + 8 * g;
+                Frag fa[MT], fb[NB];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int i = 0; i < MT; ++i) {
+                    fa[i].raw = uint4{0, 0, 0, 0};
+                    if (row_in[i] && k < K) fa[i].raw = *reinterpret_cast<const uint4*>(arow[i] + k);
+                }
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
                     fb[j].raw = uint4{0, 0, 0, 0};
                     if (col_in[j] && k < K) fb[j].raw = *reinterpret_cast<const uint4*>(wrow[j] + k);
                 }
-            } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) fa.h[i] = (row_in && k + i < K) ? arow[k + i].bits : 0;
+                for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) fb[j].h[i] = (col_in[j] && k + i < K) ? wrow[j][k + i].bits : 0;
+                    for (int j = 0; j < NB; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
             }
+        } else {
+            for (int k0 = KSPLIT ? wave * 32 : 0; k0 < K; k0 += KSPLIT ? 128 : 32) {
+                const int k = k0 + 8 * g;
+                Frag fa[MT], fb[NB];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa.v, fb[j].v, acc[j], 0, 0, 0);
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) fa[i].h[u] = (row_in[i] && k + u < K) ? arow[i][k + u].bits : 0;
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) fb[j].h[u] = (col_in[j] && k + u < K) ? wrow[j][k + u].bits : 0;
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < NB; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
+            }
         }
     } else {
         // true float32 on the matrix cores: an instruction takes four values of K, one a lane group
-        for (int k0 = 0; k0 < K; k0 += 4) {
+#pragma unroll 2
+        for (int k0 = KSPLIT ? wave * 4 : 0; k0 < K; k0 += KSPLIT ? 16 : 4) {
             const int k = k0 + g;
-            const float fa = (row_in && k < K) ? to_float(arow[k]) : 0.f;
+            float fa[MT], fb[NB];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float fb = (col_in[j] && k < K) ? to_float(wrow[j][k]) : 0.f;
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa, fb, acc[j], 0, 0, 0);
-            }
+            for (int i = 0; i < MT; ++i) fa[i] = (row_in[i] && k < K) ? to_float(arow[i][k]) : 0.f;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) fb[j] = (col_in[j] && k < K) ? to_float(wrow[j][k]) : 0.f;
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NB; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
     }
-    // accumulator register i: slot row 4 g + i, output n0 + 16 j + r
+    if constexpr (KSPLIT) {
+        if (wave > 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = 4 * g + i;
-        if (row >= n_rows) continue;
-        const int64_t slot = slot0 + row;
-        const float scale = epilogue == 1 ? pair_weight[order[slot]] : 1.f;
+            for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + 16 * j + r;
-            if (n >= N) continue;
-            const float v = acc[j][i];
-            if (epilogue == 1) static_cast<float*>(out)[slot * N + n] = v * scale;
-            else static_cast<T*>(out)[slot * N + n] = from_float<T>(gelu_erf(v));
+                for (int j = 0; j < NB; ++j)
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) red[((((wave - 1) * MT + i) * NB + j) * 4 + u) * 64 + lane] = acc[i][j][u];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int ww = 0; ww < 3; ++ww)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc[i][j][u] += red[(((ww * MT + i) * NB + j) * 4 + u) * 64 + lane];
+    }
+    // accumulator register u of block i: slot row 16 i + 4 g + u, output n0 + 16 j + r
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int row = 16 * i + 4 * g + u;
+            if (row >= n_rows) continue;
+            const int64_t slot = slot0 + row;
+            const float scale = epilogue == 1 ? pair_weight[order[slot]] : 1.f;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const int n = n0 + 16 * j + r;
+                if (n >= N) continue;
+                const float v = acc[i][j][u];
+                if (epilogue == 1) static_cast<float*>(out)[slot * N + n] = v * scale;
+                else static_cast<T*>(out)[slot * N + n] = from_float<T>(gelu_erf(v));
+            }
         }
     }
 }
@@ -280,22 +374,36 @@ extern "C" int fsie_moe_group(const int32_t* ids, int n_pairs, int experts, int 
     return 0;
 }
 
+// Rows of a tile that the products are best run with for this many (token, choice) pairs over this many experts: 16
+// (the weights' read bounds the product: the waves split K), 64 or 128 (a weight fragment serves four or eight
+// blocks of rows).  fsie_moe_group and fsie_moe_gemm take any of the three.
+extern "C" int fsie_moe_tile_rows(int n_pairs, int experts) {
+    const int per_expert = n_pairs / (experts > 0 ? experts : 1);
+    return per_expert >= 256 ? 128 : per_expert >= 48 ? 64 : 16;
+}
+
 extern "C" int fsie_moe_gemm(const void* a, const void* w, void* out, const int32_t* tiles, int max_tiles,
                              const int32_t* order, int gather_div, const float* pair_weight, int N, int K, int epilogue,
                              int dtype, int tile_rows, hipStream_t stream) {
     FSIE_REQUIRE(max_tiles >= 0 && N > 0 && K > 0 && gather_div >= 0, "moe_gemm: bad sizes tiles=%d N=%d K=%d", max_tiles, N, K);
-    FSIE_REQUIRE(tile_rows == kTileRows, "moe_gemm: tiles of %d rows (the kernel takes %d)", tile_rows, kTileRows);
+    FSIE_REQUIRE(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_gemm: tiles of %d rows (the kernels take 16, 64, 128)",
+                 tile_rows);
     FSIE_REQUIRE(a && w && out && tiles && order, "moe_gemm: missing operand");
     FSIE_REQUIRE(epilogue == 0 || (epilogue == 1 && pair_weight), "moe_gemm: unknown epilogue %d", epilogue);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "moe_gemm: unknown dtype %d", dtype);
     if (max_tiles == 0) return 0;
-    const dim3 grid(static_cast<unsigned>(max_tiles), static_cast<unsigned>((N + 255) / 256));
-    if (dtype == FSIE_F32)
-        moe_gemm_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(a), static_cast<const float*>(w), out, tiles,
-                                                         order, gather_div, pair_weight, N, K, epilogue);
-    else
-        moe_gemm_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, tiles,
-                                                          order, gather_div, pair_weight, N, K, epilogue);
+#define FSIE_MOE_GEMM(T, MT, NB, KSPLIT)                                                                                 \
+    moe_gemm_kernel<T, MT, NB, KSPLIT><<<dim3(static_cast<unsigned>(max_tiles),                                           \
+                                              static_cast<unsigned>(ceil_div64(N, KSPLIT ? 16 * NB : 64 * NB))),           \
+                                         256, 0, stream>>>(static_cast<const T*>(a), static_cast<const T*>(w), out, tiles, order, \
+                                                           gather_div, pair_weight, N, K, epilogue)
+#define FSIE_MOE_GEMM_T(T)                                      \
+    if (tile_rows == 16) FSIE_MOE_GEMM(T, 1, 2, true);          \
+    else if (tile_rows == 64) FSIE_MOE_GEMM(T, 4, 4, false);    \
+    else FSIE_MOE_GEMM(T, 8, 4, false)
+    if (dtype == FSIE_F32) { FSIE_MOE_GEMM_T(float); } else { FSIE_MOE_GEMM_T(bf16_t); }
+#undef FSIE_MOE_GEMM_T
+#undef FSIE_MOE_GEMM
     FSIE_CHECK_LAUNCH("moe_gemm");
     return 0;
 }

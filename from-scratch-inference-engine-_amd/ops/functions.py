@@ -1088,11 +1088,14 @@ def mlstm_state_floats(dim: int, vdim: int) -> int:
 
 
 def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: torch.Tensor, gate_cap: float, q_scale: float,
-               state: torch.Tensor, q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int):
+               state: torch.Tensor, q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int,
+               chunked: bool = True):
     """The matrix memory over the step's tokens, request by request in order.  ``proj`` [T, W] holds q, k (heads * dim
     each) and v (heads * vdim) at their column offsets; ``gates`` float32 [T, 2 * heads]: the input gates' logits, then
     the forget gates'; ``state`` float32 [slots, heads, mlstm_state_floats(dim, vdim)], updated in place.  Returns
-    (num [T, heads, vdim], den [T, heads], coef [T, heads, 4]), all float32: S^T q, n . q and (keep, take, exp(-m), m)."""
+    (num [T, heads, vdim], den [T, heads], coef [T, heads, 4]), all float32: S^T q, n . q and (f, i, m before the token,
+    m).  Long portions are computed chunk by chunk on the matrix cores (the same sums in another order);
+    ``chunked=False`` walks every portion token by token."""
     _need(proj, "mlstm proj", ndim=2)
     t, w = proj.shape
     if max(q_off + heads * dim, k_off + heads * dim, v_off + heads * vdim) > w:
@@ -1106,10 +1109,20 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gates: to
     num = torch.empty((t, heads, vdim), dtype=torch.float32, device=proj.device)
     den = torch.empty((t, heads), dtype=torch.float32, device=proj.device)
     coef = torch.empty((t, heads, 4), dtype=torch.float32, device=proj.device)
+    n = seq_slots.shape[0]
+    if q_starts.shape[0] != n + 1:
+        raise KernelError("mlstm_scan: q_starts must have one entry more than seq_slots")
+    chunk_tokens, chunk_min, chunk_floats = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int64(0)
+    check(load().fsie_mlstm_scan_shape(heads, dim, vdim, ctypes.byref(chunk_tokens), ctypes.byref(chunk_min),
+                                       ctypes.byref(chunk_floats)))
+    # a step of single tokens (t == n, as every captured decode step is) has no portion to cut into chunks
+    max_chunks = t // chunk_tokens.value + n if chunked and chunk_floats.value and t > n and t >= chunk_min.value else 0
+    work = torch.empty((max_chunks * chunk_floats.value,), dtype=torch.float32, device=proj.device) if max_chunks else None
     check(load().fsie_mlstm_scan(proj.data_ptr(), w, q_off, k_off, v_off, dtype_code(proj.dtype), gates.data_ptr(),
                                  float(gate_cap), float(q_scale), state.data_ptr(), state.shape[0], q_starts.data_ptr(),
-                                 seq_slots.data_ptr(), seq_slots.shape[0], t, heads, dim, vdim, coef.data_ptr(),
-                                 num.data_ptr(), den.data_ptr(), _stream()))
+                                 seq_slots.data_ptr(), n, t, heads, dim, vdim, coef.data_ptr(),
+                                 num.data_ptr(), den.data_ptr(), work.data_ptr() if work is not None else None, max_chunks,
+                                 _stream()))
     return num, den, coef
 
 

@@ -97,7 +97,8 @@ _SIGNATURES = {
     "fsie_causal_conv": ([_P, _P, _P, _P, c_int64, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_mlstm_state_floats": ([c_int, c_int], c_int64),
     "fsie_mlstm_scan": ([_P, c_int64, c_int, c_int, c_int, c_int, _P, c_float, c_float, _P, c_int, _P, _P, c_int, c_int, c_int,
-                         c_int, c_int, _P, _P, _P, _P], c_int),
+                         c_int, c_int, _P, _P, _P, _P, c_int, _P], c_int),
+    "fsie_mlstm_scan_shape": ([c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int64)], c_int),
     "fsie_mlstm_out": ([_P, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_moe_route": ([_P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_float, _P], c_int),
     "fsie_moe_group": ([_P, c_int, c_int, c_int, _P, _P, _P, c_int, _P], c_int),
