@@ -253,12 +253,15 @@ int fsie_group_rmsnorm(float* residual, const void* delta1, int delta1_dtype, co
 // ---- a short causal convolution over time, added to its input -----------------------------------
 // y[t] = x[t] + sum_j w[:, j] * x[t - taps + 1 + j] within a request, channel by channel (w [hidden][taps], float32);
 // the inputs before a portion's first token come from state[slot] [taps - 1][hidden] (float32, oldest first; zeros
-// when the request starts), which a second kernel then brings up to date with the portion's last inputs.
-// x [n_tokens][hidden] float32, y in `dtype`; q_starts [n_seqs + 1], seq_slots [n_seqs].  `state` is the slots'
-// first record: consecutive slots lie `slot_stride` floats apart (several convolutions may share a slot).
-int fsie_causal_conv(const float* x, const float* w, void* y, float* state, int64_t slot_stride, int n_slots,
-                     const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, int hidden, int taps,
-                     int dtype, hipStream_t stream);
+// when the request starts), which is then brought up to date with the portion's last inputs (by the same kernel for
+// a request's single token, by a second kernel for longer portions).
+// x [n_tokens][hidden] float32, y in `dtype`; q_starts [n_seqs + 1], seq_slots [n_seqs]; every request of the step
+// brings at least one token.  `state` is the slots' first record: consecutive slots lie `slot_stride` floats apart
+// (several convolutions may share a slot).  x2, w2, y2 (all or none): a second convolution of the same sizes in the
+// same launches, its state `second` floats into a slot's record.
+int fsie_causal_conv(const float* x, const float* w, void* y, const float* x2, const float* w2, void* y2, float* state,
+                     int64_t slot_stride, int64_t second, int n_slots, const int32_t* q_starts, const int32_t* seq_slots,
+                     int n_seqs, int n_tokens, int hidden, int taps, int dtype, hipStream_t stream);
 
 // ---- mLSTM: a matrix memory with exponential gates ------------------------------------------------
 // gates [n_tokens][2 * heads] float32 (input gate logits, then forget gate logits); per request and head the running
@@ -294,7 +297,9 @@ int fsie_moe_group(const int32_t* ids, int n_pairs, int experts, int tile_rows, 
                    int32_t* tiles, int max_tiles, hipStream_t stream);
 // One product per expert over its tiles: out[slot] = epilogue(A[row(slot)] . W[expert]^T), W [experts][N][K] in `dtype`.
 // gather_div > 0: row(slot) = order[slot] / gather_div (rows of A are tokens); 0: row(slot) = slot.
-// epilogue 0: exact GELU, out in `dtype`; 1: times slot_weight[order[slot]], out float32.
+// epilogue 0: exact GELU, out in `dtype`; 1: times slot_weight[order[slot]], out float32.  tile_rows: 16, 64 or 128,
+// the rows of a tile of `tiles`; fsie_moe_tile_rows names the one that suits a step of n_pairs pairs.
+int fsie_moe_tile_rows(int n_pairs, int experts);
 int fsie_moe_gemm(const void* a, const void* w, void* out, const int32_t* tiles, int max_tiles, const int32_t* order,
                   int gather_div, const float* pair_weight, int N, int K, int epilogue, int dtype, int tile_rows,
                   hipStream_t stream);

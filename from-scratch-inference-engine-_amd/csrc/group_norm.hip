@@ -61,55 +61,72 @@ __global__ __launch_bounds__(kThreads) void group_rmsnorm_kernel(
     }
 }
 
+// One workgroup a token, for one convolution or for a layer's two (x, w, y and the state of the second follow the
+// first's: `second` floats into a slot's record).  A request that brings a single token has its state brought up to
+// date here, by the threads that have just read it (a thread owns its channels); longer portions leave that to the
+// second kernel, which runs after every row has been written.
 template <typename T>
-__global__ __launch_bounds__(kThreads) void causal_conv_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                               T* __restrict__ y, const float* __restrict__ state,
-                                                               int64_t slot_stride, int n_slots,
+__global__ __launch_bounds__(kThreads) void causal_conv_kernel(const float* __restrict__ xa, const float* __restrict__ xb,
+                                                               const float* __restrict__ wa, const float* __restrict__ wb,
+                                                               T* __restrict__ ya, T* __restrict__ yb, float* __restrict__ state,
+                                                               int64_t slot_stride, int64_t second, int n_slots,
                                                                const int32_t* __restrict__ q_starts,
                                                                const int32_t* __restrict__ seq_slots, int n_seqs, int hidden,
                                                                int taps) {
-    __shared__ int s_info[2];
+    __shared__ int s_info[3];
     const int t = blockIdx.x;
-    if (threadIdx.x == 0) {
-        // the request of this row: the last one whose first row is not beyond it
-        int lo = 0, hi = n_seqs - 1;
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (q_starts[mid] <= t) lo = mid; else hi = mid - 1;
+    // the request of this row: the one whose rows begin at or before it and end after it (every thread tries one)
+    for (int s = threadIdx.x; s < n_seqs; s += kThreads) {
+        const int lo = q_starts[s], hi = q_starts[s + 1];
+        if (lo <= t && t < hi) {
+            const int slot = seq_slots[s];
+            s_info[0] = lo;
+            s_info[1] = (slot >= 0 && slot < n_slots) ? slot : -1;
+            s_info[2] = hi - lo;
         }
-        const int slot = seq_slots[lo];
-        s_info[0] = q_starts[lo];
-        s_info[1] = (slot >= 0 && slot < n_slots) ? slot : -1;
     }
     __syncthreads();
     const int first = s_info[0], slot = s_info[1];
-    const float* st = slot >= 0 ? state + slot * slot_stride : nullptr;
-    for (int c = threadIdx.x; c < hidden; c += kThreads) {
-        const float here = x[static_cast<int64_t>(t) * hidden + c];
-        float acc = here;
-        for (int j = 0; j < taps; ++j) {
-            const int back = taps - 1 - j;  // how many tokens before this one
-            const int src = t - back;
-            float v;
-            if (src >= first) v = back ? x[static_cast<int64_t>(src) * hidden + c] : here;
-            else v = st ? st[static_cast<int64_t>(taps - 1 - (first - src)) * hidden + c] : 0.f;  // state row taps-1-k = k tokens before the portion
-            acc = fmaf(w[c * taps + j], v, acc);
+    const bool store = s_info[2] == 1 && slot >= 0 && taps > 1;
+    const int keep = taps - 1;
+    for (int which = 0; which < (xb ? 2 : 1); ++which) {
+        const float* x = which ? xb : xa;
+        const float* w = which ? wb : wa;
+        T* y = which ? yb : ya;
+        float* st = slot >= 0 ? state + slot * slot_stride + which * second : nullptr;
+        for (int c = threadIdx.x; c < hidden; c += kThreads) {
+            const float here = x[static_cast<int64_t>(t) * hidden + c];
+            float acc = here;
+            for (int j = 0; j < taps; ++j) {
+                const int back = taps - 1 - j;  // how many tokens before this one
+                const int src = t - back;
+                float v;
+                if (src >= first) v = back ? x[static_cast<int64_t>(src) * hidden + c] : here;
+                else v = st ? st[static_cast<int64_t>(keep - (first - src)) * hidden + c] : 0.f;  // state row keep - k = k tokens before the portion
+                acc = fmaf(w[c * taps + j], v, acc);
+                // (a single token: src < first for every back > 0, and row keep - back moves one row up)
+                if (store && back > 0 && back < keep) st[static_cast<int64_t>(keep - back - 1) * hidden + c] = v;
+            }
+            if (store) st[static_cast<int64_t>(keep - 1) * hidden + c] = here;
+            y[static_cast<int64_t>(t) * hidden + c] = from_float<T>(acc);
         }
-        y[static_cast<int64_t>(t) * hidden + c] = from_float<T>(acc);
     }
 }
 
-// state'[i] for i in [0, taps - 1): the input (taps - 1 - i) tokens before the next portion's first token
-__global__ __launch_bounds__(kThreads) void causal_conv_store_kernel(const float* __restrict__ x, float* __restrict__ state,
-                                                                     int64_t slot_stride, int n_slots,
+// state'[i] for i in [0, taps - 1): the input (taps - 1 - i) tokens before the next portion's first token.
+// grid = (requests, convolutions); a request of one token has been dealt with already.
+__global__ __launch_bounds__(kThreads) void causal_conv_store_kernel(const float* __restrict__ xa, const float* __restrict__ xb,
+                                                                     float* __restrict__ state, int64_t slot_stride,
+                                                                     int64_t second, int n_slots,
                                                                      const int32_t* __restrict__ q_starts,
                                                                      const int32_t* __restrict__ seq_slots, int hidden,
                                                                      int taps) {
     const int s = blockIdx.x;
     const int slot = seq_slots[s];
     const int first = q_starts[s], n = q_starts[s + 1] - first;
-    if (slot < 0 || slot >= n_slots || n <= 0) return;
-    float* st = state + slot * slot_stride;
+    if (slot < 0 || slot >= n_slots || n <= 1) return;
+    const float* x = blockIdx.y ? xb : xa;
+    float* st = state + slot * slot_stride + blockIdx.y * second;
     const int keep = taps - 1;
     for (int c = threadIdx.x; c < hidden; c += kThreads) {
         // a thread owns its channel: old rows are read before they are overwritten (ascending i reads row i + n >= i)
@@ -165,24 +182,32 @@ extern "C" int fsie_group_rmsnorm(float* residual, const void* delta1, int delta
     return 0;
 }
 
-extern "C" int fsie_causal_conv(const float* x, const float* w, void* y, float* state, int64_t slot_stride, int n_slots,
-                                const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, int hidden,
-                                int taps, int dtype, hipStream_t stream) {
+// x2 (with w2, y2): a second convolution of the same sizes in the same launches; its state lies `second` floats into a
+// slot's record.
+extern "C" int fsie_causal_conv(const float* x, const float* w, void* y, const float* x2, const float* w2, void* y2,
+                                float* state, int64_t slot_stride, int64_t second, int n_slots, const int32_t* q_starts,
+                                const int32_t* seq_slots, int n_seqs, int n_tokens, int hidden, int taps, int dtype,
+                                hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && hidden > 0 && taps >= 1 && n_slots > 0,
                  "causal_conv: bad sizes T=%d requests=%d hidden=%d taps=%d", n_tokens, n_seqs, hidden, taps);
     FSIE_REQUIRE(x && w && y && q_starts && seq_slots && (taps == 1 || state), "causal_conv: missing operand");
-    FSIE_REQUIRE(slot_stride >= static_cast<int64_t>(taps - 1) * hidden, "causal_conv: slots closer than a state is long");
+    FSIE_REQUIRE((!x2) == (!w2) && (!x2) == (!y2), "causal_conv: a second convolution comes with its weights and its result");
+    const int64_t one = static_cast<int64_t>(taps - 1) * hidden;
+    FSIE_REQUIRE(slot_stride >= (x2 ? second + one : one) && (!x2 || second >= one), "causal_conv: slots closer than a state is long");
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "causal_conv: unknown dtype %d", dtype);
     if (n_tokens == 0 || n_seqs == 0) return 0;
     if (dtype == FSIE_F32)
-        causal_conv_kernel<float><<<n_tokens, kThreads, 0, stream>>>(x, w, static_cast<float*>(y), state, slot_stride, n_slots,
-                                                                     q_starts, seq_slots, n_seqs, hidden, taps);
+        causal_conv_kernel<float><<<n_tokens, kThreads, 0, stream>>>(x, x2, w, w2, static_cast<float*>(y), static_cast<float*>(y2),
+                                                                     state, slot_stride, second, n_slots, q_starts, seq_slots,
+                                                                     n_seqs, hidden, taps);
     else
-        causal_conv_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(x, w, static_cast<bf16_t*>(y), state, slot_stride, n_slots,
-                                                                      q_starts, seq_slots, n_seqs, hidden, taps);
+        causal_conv_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(x, x2, w, w2, static_cast<bf16_t*>(y), static_cast<bf16_t*>(y2),
+                                                                      state, slot_stride, second, n_slots, q_starts, seq_slots,
+                                                                      n_seqs, hidden, taps);
     FSIE_CHECK_LAUNCH("causal_conv");
-    if (taps > 1) {
-        causal_conv_store_kernel<<<n_seqs, kThreads, 0, stream>>>(x, state, slot_stride, n_slots, q_starts, seq_slots, hidden, taps);
+    if (taps > 1 && n_tokens != n_seqs) {  // (as many tokens as requests: one each, or the kernel above would have no request for a row)
+        causal_conv_store_kernel<<<dim3(n_seqs, x2 ? 2 : 1), kThreads, 0, stream>>>(x, x2, state, slot_stride, second, n_slots,
+                                                                                   q_starts, seq_slots, hidden, taps);
         FSIE_CHECK_LAUNCH("causal_conv_store");
     }
     return 0;

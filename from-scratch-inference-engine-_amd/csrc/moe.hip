@@ -151,9 +151,28 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restri
             tl[0] = e, tl[1] = first, tl[2] = min(tile_rows, s_start[e + 1] - first);
         }
     }
+    __shared__ int s_scan[1024];
+    if (n_pairs <= static_cast<int>(blockDim.x)) {
+        // a pair a thread at most (every decode step): the pairs of its expert before it are counted one by one, all
+        // threads reading the same id at a time
+        int mine = -1;
+        if (tid < n_pairs) {
+            mine = ids[tid];
+            mine = (mine < 0 || mine >= experts) ? 0 : mine;
+        }
+        s_scan[tid] = mine;
+        __syncthreads();
+        if (tid < n_pairs) {
+            int before = 0;
+            for (int p = 0; p < tid; ++p) before += s_scan[p] == mine;
+            const int at = s_start[mine] + before;
+            order[at] = tid;
+            slot_of[tid] = at;
+        }
+        return;
+    }
     // pass 2: a pair's slot = its expert's start + the pairs of that expert before it.  An expert at a time: the
     // threads' counts of it, an exclusive scan over the threads (in LDS), then the slots.
-    __shared__ int s_scan[1024];
     for (int e = 0; e < experts; ++e) {
         if (s_count[e] == 0) continue;  // (the same for all threads)
         int mine = 0;

@@ -1059,27 +1059,46 @@ def group_rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, grou
 
 
 def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, q_starts: torch.Tensor, seq_slots: torch.Tensor,
-                out_dtype: torch.dtype) -> torch.Tensor:
+                out_dtype: torch.dtype, x2: Optional[torch.Tensor] = None, weight2: Optional[torch.Tensor] = None,
+                state2: Optional[torch.Tensor] = None):
     """``x + conv(x)``: a causal convolution over time within every request, channel by channel.  ``x`` float32 [T, H];
     ``weight`` float32 [H, taps], the last tap on the token itself; ``state`` float32 [slots, ..., taps - 1, H], a view
     whose first dimension are the requests' slots: the inputs before a portion's first token (oldest first), brought
-    up to date by this call.  The result has ``out_dtype``."""
+    up to date by this call.  The result has ``out_dtype``.  With ``x2``, ``weight2`` and ``state2`` (a view of the
+    same slots' records, behind ``state``) a second convolution of the same sizes goes through the same launches, and
+    the result is the pair."""
     _need(x, "causal_conv x", dtype=torch.float32, ndim=2)
     t, h = x.shape
     _need(weight, "causal_conv weight", dtype=torch.float32, ndim=2)
     taps = weight.shape[1]
     if weight.shape[0] != h or taps < 1:
         raise KernelError(f"causal_conv: weight {tuple(weight.shape)} does not fit rows of {h}")
-    if taps > 1 and (not isinstance(state, torch.Tensor) or not state.is_cuda or state.dtype != torch.float32 or state.ndim != 3
-                     or tuple(state.shape[1:]) != (taps - 1, h) or state.stride(2) != 1 or state.stride(1) != h):
+
+    def state_ok(st):
+        return (isinstance(st, torch.Tensor) and st.is_cuda and st.dtype == torch.float32 and st.ndim == 3
+                and tuple(st.shape[1:]) == (taps - 1, h) and st.stride(2) == 1 and st.stride(1) == h)
+
+    if taps > 1 and not state_ok(state):
         raise KernelError(f"causal_conv: the state must be float32 [slots, {taps - 1}, {h}] with contiguous records")
     _need(q_starts, "causal_conv q_starts", dtype=torch.int32, ndim=1)
     _need(seq_slots, "causal_conv seq_slots", dtype=torch.int32, ndim=1)
     y = torch.empty((t, h), dtype=out_dtype, device=x.device)
-    check(load().fsie_causal_conv(x.data_ptr(), weight.data_ptr(), y.data_ptr(), state.data_ptr() if taps > 1 else None,
-                                  state.stride(0) if taps > 1 else 0, state.shape[0] if taps > 1 else 1, q_starts.data_ptr(), seq_slots.data_ptr(), seq_slots.shape[0], t, h, taps,
-                                  dtype_code(out_dtype), _stream()))
-    return y
+    y2, second = None, 0
+    if x2 is not None:
+        _need(x2, "causal_conv x2", dtype=torch.float32, shape=(t, h))
+        _need(weight2, "causal_conv weight2", dtype=torch.float32, shape=(h, taps))
+        if taps > 1:
+            if not state_ok(state2) or state2.stride(0) != state.stride(0) or state2.shape[0] != state.shape[0]:
+                raise KernelError("causal_conv: the second state must be a view of the same slots' records")
+            second = (state2.data_ptr() - state.data_ptr()) // 4
+            if second < (taps - 1) * h or second + (taps - 1) * h > state.stride(0):
+                raise KernelError("causal_conv: the second state must lie behind the first in a slot's record")
+        y2 = torch.empty((t, h), dtype=out_dtype, device=x.device)
+    check(load().fsie_causal_conv(x.data_ptr(), weight.data_ptr(), y.data_ptr(), _ptr(x2), _ptr(weight2), _ptr(y2),
+                                  state.data_ptr() if taps > 1 else None, state.stride(0) if taps > 1 else 2 * max(taps - 1, 0) * h,
+                                  second, state.shape[0] if taps > 1 else 1, q_starts.data_ptr(), seq_slots.data_ptr(),
+                                  seq_slots.shape[0], t, h, taps, dtype_code(out_dtype), _stream()))
+    return y if x2 is None else (y, y2)
 
 
 def mlstm_state_floats(dim: int, vdim: int) -> int:
@@ -1144,7 +1163,9 @@ def mlstm_out(num: torch.Tensor, den: torch.Tensor, coef: torch.Tensor, gate: to
     return y
 
 
-MOE_TILE_ROWS = 16
+def moe_tile_rows(n_pairs: int, experts: int) -> int:
+    """Rows of a tile of the experts' products for a step of this many (token, choice) pairs: 16, 64 or 128."""
+    return int(load().fsie_moe_tile_rows(int(n_pairs), int(experts)))
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int, scale: float):
@@ -1165,27 +1186,29 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, t
     return ids, weights
 
 
-def moe_group(ids: torch.Tensor, experts: int):
+def moe_group(ids: torch.Tensor, experts: int, tile_rows: Optional[int] = None):
     """The (token, choice) pairs of ``ids`` [T, top] grouped by expert: (order int32 [pairs]: the pair in every slot,
-    slot_of int32 [pairs], tiles int32 [max_tiles, 3]: (expert, first slot, slots) of every tile of MOE_TILE_ROWS
-    slots; unused tiles have no slots)."""
+    slot_of int32 [pairs], tiles int32 [max_tiles, 3]: (expert, first slot, slots) of every tile of ``tile_rows``
+    slots (default: what ``moe_tile_rows`` names for the step); unused tiles have no slots)."""
     _need(ids, "moe_group ids", dtype=torch.int32, ndim=2)
     n = ids.numel()
-    max_tiles = -(-n // MOE_TILE_ROWS) + experts
+    tile_rows = moe_tile_rows(n, experts) if tile_rows is None else int(tile_rows)
+    max_tiles = -(-n // tile_rows) + experts
     order = torch.empty((n,), dtype=torch.int32, device=ids.device)
     slot_of = torch.empty((n,), dtype=torch.int32, device=ids.device)
     tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=ids.device)
-    check(load().fsie_moe_group(ids.data_ptr(), n, int(experts), MOE_TILE_ROWS, order.data_ptr(), slot_of.data_ptr(),
+    check(load().fsie_moe_group(ids.data_ptr(), n, int(experts), tile_rows, order.data_ptr(), slot_of.data_ptr(),
                                 tiles.data_ptr(), max_tiles, _stream()))
     return order, slot_of, tiles
 
 
 def moe_gemm(a: torch.Tensor, weight: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, gather_div: int = 0,
-             pair_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+             pair_weight: Optional[torch.Tensor] = None, tile_rows: Optional[int] = None) -> torch.Tensor:
     """One product per expert: out[slot] = a[row(slot)] . weight[expert of slot]^T with ``weight`` [E, N, K].
     ``gather_div`` > 0: row(slot) = order[slot] // gather_div (``a`` holds tokens); 0: row(slot) = slot.  Without
     ``pair_weight`` the result is the exact GELU of the product in ``a``'s type; with it (float32 [pairs]) the product
-    times the pair's weight, float32."""
+    times the pair's weight, float32.  ``tile_rows``: the rows of a tile of ``tiles`` (default: what ``moe_tile_rows``
+    names for the step, as ``moe_group``'s default is)."""
     _need(a, "moe_gemm a", ndim=2)
     _need(weight, "moe_gemm weight", dtype=a.dtype, ndim=3)
     _, n, k = weight.shape
@@ -1194,6 +1217,7 @@ def moe_gemm(a: torch.Tensor, weight: torch.Tensor, tiles: torch.Tensor, order: 
     _need(tiles, "moe_gemm tiles", dtype=torch.int32, ndim=2)
     _need(order, "moe_gemm order", dtype=torch.int32, ndim=1)
     slots = order.shape[0]
+    tile_rows = moe_tile_rows(slots, weight.shape[0]) if tile_rows is None else int(tile_rows)
     if not gather_div and a.shape[0] != slots:
         raise KernelError("moe_gemm: without a gather the rows are the slots")
     if pair_weight is not None:
@@ -1203,7 +1227,7 @@ def moe_gemm(a: torch.Tensor, weight: torch.Tensor, tiles: torch.Tensor, order: 
     out = torch.empty((slots, n), dtype=torch.float32 if pair_weight is not None else a.dtype, device=a.device)
     check(load().fsie_moe_gemm(a.data_ptr(), weight.data_ptr(), out.data_ptr(), tiles.data_ptr(), tiles.shape[0],
                                order.data_ptr(), int(gather_div), _ptr(pair_weight), n, k, 1 if pair_weight is not None else 0,
-                               dtype_code(a.dtype), MOE_TILE_ROWS, _stream()))
+                               dtype_code(a.dtype), tile_rows, _stream()))
     return out
 
 

@@ -94,7 +94,8 @@ _SIGNATURES = {
     "fsie_gate_heads": ([_P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_group_rmsnorm": ([_P, _P, c_int, _P, c_int, c_float, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int,
                             _P], c_int),
-    "fsie_causal_conv": ([_P, _P, _P, _P, c_int64, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_causal_conv": ([_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+                         c_int),
     "fsie_mlstm_state_floats": ([c_int, c_int], c_int64),
     "fsie_mlstm_scan": ([_P, c_int64, c_int, c_int, c_int, c_int, _P, c_float, c_float, _P, c_int, _P, _P, c_int, c_int, c_int,
                          c_int, c_int, _P, _P, _P, _P, c_int, _P], c_int),
@@ -103,6 +104,7 @@ _SIGNATURES = {
     "fsie_moe_route": ([_P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_float, _P], c_int),
     "fsie_moe_group": ([_P, c_int, c_int, c_int, _P, _P, _P, c_int, _P], c_int),
     "fsie_moe_gemm": ([_P, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_moe_tile_rows": ([c_int, c_int], c_int),
     "fsie_moe_combine": ([_P, _P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_sample": ([_P, c_int, c_int, _P, _P, _P, _P, _P, _P], c_int),
 }

@@ -129,8 +129,15 @@ class ParallelBlock(Block):
         else:
             a = self.mixer_norm(hidden, a_type)  # (adds the pending deltas; the second norm then finds none)
             b = self.ffn_norm(hidden, b_type)
-        a = self._conv(self.mixer_conv, a, ctx, state)
-        b = self._conv(self.ffn_conv, b, ctx, state)
+        pair = getattr(self.mixer_conv, "forward_pair", None)
+        if (pair is not None and type(self.ffn_conv) is type(self.mixer_conv) and 0 not in self.mixer_conv.state_shape()
+                and self.mixer_conv.state_shape() == self.ffn_conv.state_shape()):
+            if state is None or state.state is None:
+                raise RuntimeError("parallel block: no state for its convolutions (the model did not ask for the block's need)")
+            a, b = pair(a, state.state[:, 0], self.ffn_conv, b, state.state[:, 1], ctx)  # two convolutions, one pass
+        else:
+            a = self._conv(self.mixer_conv, a, ctx, state)
+            b = self._conv(self.ffn_conv, b, ctx, state)
         hidden.delta = self.mixer.forward(a, ctx, cache)
         hidden.delta2 = self.ffn.forward(b, ctx)
         hidden.delta_scale = self.residual_scale

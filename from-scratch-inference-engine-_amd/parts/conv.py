@@ -33,3 +33,8 @@ class CausalResidualConvolution(Convolution):
 
     def forward(self, x: torch.Tensor, ctx, state: torch.Tensor) -> torch.Tensor:
         return ops.causal_conv(x, self.weight, state, ctx.q_starts, ctx.seq_slots, ctx.compute_dtype)
+
+    def forward_pair(self, x: torch.Tensor, state: torch.Tensor, other: "CausalResidualConvolution", x2: torch.Tensor,
+                     state2: torch.Tensor, ctx):
+        """This convolution of ``x`` and ``other`` (of the same sizes) of ``x2`` in the same kernels."""
+        return ops.causal_conv(x, self.weight, state, ctx.q_starts, ctx.seq_slots, ctx.compute_dtype, x2, other.weight, state2)

@@ -384,7 +384,7 @@ def test_matrix_memory_output_norm_and_gate(ops, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("t, hidden, ff, experts, top", [(50, 64, 96, 8, 3), (7, 90, 34, 5, 5), (300, 40, 17, 3, 1), (1, 32, 32, 1, 1),
-                                                         (130, 128, 272, 16, 2)])
+                                                         (130, 128, 272, 16, 2), (600, 48, 40, 2, 1)])
 def test_routed_experts_against_the_plain_ones(ops, dtype, t, hidden, ff, experts, top):
     """Router (corrections that move the choice and leave the weights alone), grouping, both products and the sum,
     as the part does them, at sizes that are multiples of nothing."""
@@ -418,9 +418,40 @@ def test_routed_experts_against_the_plain_ones(ops, dtype, t, hidden, ff, expert
     assert (np.diff(flat[order]) >= 0).all()  # slots of an expert are consecutive
     covered = np.zeros(t * top, dtype=int)
     for e, first, n in tiles:
-        assert 0 <= n <= 16 and (n == 0 or (flat[order[first:first + n]] == e).all())
+        assert 0 <= n <= ops.moe_tile_rows(t * top, experts) and (n == 0 or (flat[order[first:first + n]] == e).all())
         covered[first:first + n] += 1
     assert (covered == 1).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_experts_products_do_not_depend_on_the_tiles(ops, dtype):
+    """Tiles of 16, 64 and 128 rows (a few rows an expert, many, very many) over the same pairs: the same products
+    up to the order of their sums, whichever expert is crowded or empty, at sizes that are multiples of nothing."""
+    t, top, n_experts, hidden, ff = 333, 2, 5, 72, 50
+    assert [ops.moe_tile_rows(n, 8) for n in (16, 8 * 47, 8 * 48, 8 * 255, 8 * 256)] == [16, 16, 64, 64, 128]
+    x = rnd((t, hidden), 1).to(dtype).cuda()
+    up = rnd((n_experts, ff, hidden), 2, hidden ** -0.5).to(dtype).cuda()
+    down = rnd((n_experts, hidden, ff), 3, ff ** -0.5).to(dtype).cuda()
+    ids = torch.randint(0, n_experts - 1, (t, top), generator=torch.Generator().manual_seed(4), dtype=torch.int32)  # the last: empty
+    ids[:200, 0] = 1  # a crowded one
+    weights = rnd((t * top,), 5).abs().cuda()
+    got = {}
+    for rows in (16, 64, 128):
+        order, slot_of, tiles = ops.moe_group(ids.cuda(), n_experts, tile_rows=rows)
+        act = ops.moe_gemm(x, up, tiles, order, gather_div=top, tile_rows=rows)
+        out = ops.moe_gemm(act, down, tiles, order, pair_weight=weights, tile_rows=rows)
+        got[rows] = ops.moe_combine(out, slot_of, t, top).cpu().double().numpy()
+    xs, e = x.cpu().double().numpy(), ids.numpy()
+    ref = np.zeros((t, hidden))
+    for i in range(t):
+        for c in range(top):
+            hid = plain.gelu_erf(up[e[i, c]].cpu().double().numpy() @ xs[i])
+            if dtype == torch.bfloat16:
+                hid = torch.tensor(hid).to(dtype).double().numpy()
+            ref[i] += float(weights[i * top + c]) * (down[e[i, c]].cpu().double().numpy() @ hid)
+    for rows in (16, 64, 128):
+        assert rel(got[rows], ref) <= tol(dtype, 2e-5, 2.0 ** -6), rows
+        assert rel(got[rows], got[16]) <= tol(dtype, 2e-6, 2.0 ** -7), rows
 
 
 # ------------------------------------------------------------------------------------------------
