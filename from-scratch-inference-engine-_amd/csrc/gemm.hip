@@ -8,6 +8,7 @@
 // A row's sum order depends on K only, never on how many other rows the call has.
 #include "common.h"
 #include "api.h"
+#include "wave_dots.h"
 
 namespace {
 
@@ -207,14 +208,49 @@ int launch_skinny(const void* x, const void* w, const float* bias, void* y, int 
     return launch_skinny_mt<T, OutT, 8>(x, w, bias, y, M, N, K, stream);
 }
 
+// Few outputs a row (gates, routers): a wave a row of x, float32 results; the matrix stays in cache.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_narrow_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                          const float* __restrict__ bias, float* __restrict__ y, int M, int N,
+                                                          int K) {
+    const int lane = threadIdx.x & 63;
+    const int m = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (m >= M) return;
+    const T* row = x + static_cast<int64_t>(m) * K;
+    const bool vec = wave_dots_vec(x, w, K);
+    for (int n0 = 0; n0 < N; n0 += kWaveDots) {
+        float z[kWaveDots];
+        wave_dots(row, w, K, n0, N, vec, lane, z);
+        float mine = 0.f;
+#pragma unroll
+        for (int i = 0; i < kWaveDots; ++i)
+            if (lane == i) mine = z[i];
+        if (lane < kWaveDots && n0 + lane < N) y[static_cast<int64_t>(m) * N + n0 + lane] = mine + (bias ? bias[n0 + lane] : 0.f);
+    }
+}
+
 }  // namespace
 
-// kind: 0 = choose by M, 1 = tiled, 2 = skinny (M <= 8).  out_f32: write float32 whatever dtype.
+// kind: 0 = choose by M, 1 = tiled, 2 = skinny (M <= 8), 3 = narrow (few outputs a row, float32 results: with
+// out_f32 or float32 operands).  out_f32: write float32 whatever dtype.
 extern "C" int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
                          int dtype, int out_f32, int kind, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gemm: unknown dtype %d", dtype);
-    FSIE_REQUIRE(kind >= 0 && kind <= 2, "gemm: unknown kind %d", kind);
+    FSIE_REQUIRE(kind >= 0 && kind <= 3, "gemm: unknown kind %d", kind);
+    if (kind == 3) {
+        FSIE_REQUIRE(out_f32 || dtype == FSIE_F32, "gemm: the narrow kernel writes float32");
+        if (M == 0) return 0;
+        const unsigned grid = static_cast<unsigned>((M + 3) / 4);
+        if (dtype == FSIE_F32)
+            gemm_narrow_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x), static_cast<const float*>(w), bias,
+                                                                static_cast<float*>(y), M, N, K);
+        else
+            gemm_narrow_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias,
+                                                                 static_cast<float*>(y), M, N, K);
+        FSIE_CHECK_LAUNCH("gemm_narrow");
+        return 0;
+    }
     FSIE_REQUIRE(!(kind == 2 && M > FSIE_GEMM_SKINNY_MAX_M), "gemm: skinny kernel takes at most %d rows, got %d",
                  FSIE_GEMM_SKINNY_MAX_M, M);
     if (M == 0) return 0;

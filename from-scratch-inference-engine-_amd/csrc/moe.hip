@@ -13,6 +13,7 @@
 // Nothing here waits for the host: the tile table has a fixed worst-case length and unused tiles are empty.
 #include "common.h"
 #include "api.h"
+#include "wave_dots.h"
 
 namespace {
 
@@ -22,58 +23,31 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int kMaxExperts = 256;
 constexpr int kMaxTop = 16;
 
-// The logits of kRouteGroup experts at a time: a lane takes 16 bytes of the token's row and of every expert's row
-// per round (all of a round's loads are asked for before any is used), sums its share in the order of the rounds,
-// and the lanes' shares meet in the wave's fixed order.  Rows that are not a whole number of 16 bytes, or not
-// aligned, are read value by value, with the same sums a lane.
-constexpr int kRouteGroup = 8;
-
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router,
                                                         const float* __restrict__ correction, int32_t* __restrict__ ids,
                                                         float* __restrict__ weights, int n_tokens, int hidden, int experts,
                                                         int top, float scale) {
-    constexpr int V = 16 / sizeof(T);
-    __shared__ float s_score[4][kMaxExperts];
+    __shared__ float s_score[4][kMaxExperts], s_choice[4][kMaxExperts];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + wave;
     const bool live = t < n_tokens;
     const T* row = x + static_cast<int64_t>(live ? t : 0) * hidden;
     float* score = s_score[wave];
-    const bool vec = hidden % V == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(router) & 15) == 0;
-    for (int e0 = 0; e0 < experts && live; e0 += kRouteGroup) {
-        float z[kRouteGroup];
+    float* choice = s_choice[wave];
+    const bool vec = wave_dots_vec(x, router, hidden);
+    for (int e0 = 0; e0 < experts && live; e0 += kWaveDots) {
+        float z[kWaveDots];
+        wave_dots(row, router, hidden, e0, experts, vec, lane, z);
+        // lane i keeps expert e0 + i: its score, and what the choice goes by
+        float mine = 0.f;
 #pragma unroll
-        for (int i = 0; i < kRouteGroup; ++i) z[i] = 0.f;
-        for (int j = lane * V; j < hidden; j += 64 * V) {
-            union { uint4 raw; T v[V]; } xv, wv[kRouteGroup];
-            if (vec) {
-                xv.raw = *reinterpret_cast<const uint4*>(row + j);
-#pragma unroll
-                for (int i = 0; i < kRouteGroup; ++i) {
-                    const int e = min(e0 + i, experts - 1);  // (past the last: the last once more, dropped below)
-                    wv[i].raw = *reinterpret_cast<const uint4*>(router + static_cast<int64_t>(e) * hidden + j);
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < V; ++u) xv.v[u] = j + u < hidden ? row[j + u] : from_float<T>(0.f);
-#pragma unroll
-                for (int i = 0; i < kRouteGroup; ++i) {
-                    const int e = min(e0 + i, experts - 1);
-#pragma unroll
-                    for (int u = 0; u < V; ++u)
-                        wv[i].v[u] = j + u < hidden ? router[static_cast<int64_t>(e) * hidden + j + u] : from_float<T>(0.f);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < kRouteGroup; ++i)
-#pragma unroll
-                for (int u = 0; u < V; ++u) z[i] = fmaf(to_float(xv.v[u]), to_float(wv[i].v[u]), z[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < kRouteGroup; ++i) {
-            const float sum = wave_sum(z[i]);
-            if (lane == 0 && e0 + i < experts) score[e0 + i] = 1.0f / (1.0f + expf(-sum));
+        for (int i = 0; i < kWaveDots; ++i)
+            if (lane == i) mine = z[i];
+        if (lane < kWaveDots && e0 + lane < experts) {
+            const float sc = 1.0f / (1.0f + expf(-mine));
+            score[e0 + lane] = sc;
+            choice[e0 + lane] = sc + correction[e0 + lane];
         }
     }
     __syncthreads();
@@ -88,7 +62,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
         for (int e = 0; e < experts; ++e) {
             bool taken = false;
             for (int p = 0; p < c; ++p) taken = taken || picked[p] == e;
-            const float v = score[e] + correction[e];
+            const float v = choice[e];
             if (!taken && (best < 0 || v > best_v)) best = e, best_v = v;
         }
         picked[c] = best;

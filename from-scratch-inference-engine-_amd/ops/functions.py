@@ -20,7 +20,7 @@ GEMM_MFMA_WIDE_MAX_M = 128  # the product that shares x through LDS, on a fragme
 GEMM_MFMA_SKINNY_BEST_M = 16
 GEMM_SPLITS = (2, 4, 8)  # slices of K that the few-rows product may leave as partial sums
 GEMM_MAX_SPLITS = 16     # most slices of the product that shares x through LDS, and most that a norm adds up
-GEMM_AUTO, GEMM_TILED, GEMM_SKINNY = 0, 1, 2
+GEMM_AUTO, GEMM_TILED, GEMM_SKINNY, GEMM_NARROW = 0, 1, 2, 3
 
 
 def dtype_code(dtype: torch.dtype) -> int:

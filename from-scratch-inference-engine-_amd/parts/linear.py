@@ -27,6 +27,7 @@ class Linear:
     the order of the matrix instruction's fragments (``prepare``, ``streamed``), from which the
     sibling takes every product of up to 64 rows."""
 
+    narrow_to = 64  # float32 results of at most this many outputs from bfloat16 operands: the narrow kernel
     float32_on_matrix_cores = True  # up to 64 rows of float32: v_mfma_f32_16x16x4_f32 instead of vector FMAs
     # A bfloat16 weight of at least this many bytes is kept a second time, in the order of the matrix
     # instruction's fragments, for the engine's own products (decoding): a wave then loads 1 KB in one
@@ -95,6 +96,9 @@ class Linear:
                 return ops.gemm_mfma_fp32(x, w, bias)
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
         wants_f32 = out_dtype is not None and out_dtype != x.dtype
+        if wants_f32 and out_dtype == torch.float32 and self.out_features <= self.narrow_to:
+            # a handful of float32 outputs a row (gates): a wave a row, the matrix from cache
+            return ops.gemm(x, w, bias, out_dtype=out_dtype, kind=ops.GEMM_NARROW)
         if (wants_f32 and bias is None and (8 if self.streamed is None else 1) <= m <= GEMM_MFMA_SKINNY_MAX_M
                 and ops.gemm_mfma_wide_splits_ok(self.in_features, 1)):
             # float32 results (logits) of 8 to 64 rows: x shared through LDS; from the fragment-ordered

@@ -89,13 +89,17 @@ def test_group_rms_norm_adds_two_scaled_deltas_and_gives_two_outputs(ops, dtype,
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("taps, hidden", [(4, 40), (2, 7), (7, 300), (1, 12)])
-def test_convolution_over_portions_steps_and_slots(ops, dtype, taps, hidden):
+@pytest.mark.parametrize("pair", [False, True])
+@pytest.mark.parametrize("taps, hidden", [(4, 40), (2, 7), (7, 300), (1, 12), (3, 520)])
+def test_convolution_over_portions_steps_and_slots(ops, dtype, taps, hidden, pair):
     """Three requests fed in unequal portions (single tokens, portions shorter than the convolution is long) over
     several steps, one of them in a slot that another has used, two convolutions sharing the slots: every output is
-    the input plus the convolution over the request's own earlier inputs, zeros before its start."""
+    the input plus the convolution over the request's own earlier inputs, zeros before its start.  ``pair``: both
+    convolutions in the same launches, each with its own inputs, weights and state."""
     seqs = {"a": rnd((19, hidden), 1), "b": rnd((5, hidden), 2), "c": rnd((8, hidden), 3)}
     w = rnd((hidden, taps), 4)
+    seqs0, w0 = {r: rnd(tuple(x.shape), 10 + i) for i, (r, x) in enumerate(seqs.items())}, rnd((hidden, taps), 14)
+    got0 = {r: [] for r in seqs}
     state = torch.full((4, 2, max(taps - 1, 0), hidden), 77.0).cuda() if taps > 1 else None
     slot = {"a": 0, "b": 2, "c": 1}
     plan = [[("a", 1), ("b", 1)], [("b", 2), ("a", 2)], [("a", 1), ("b", 1)], [("a", 9), ("b", 1)], [("c", 3), ("a", 1)],
@@ -108,21 +112,48 @@ def test_convolution_over_portions_steps_and_slots(ops, dtype, taps, hidden):
                 slot["c"] = slot["b"]  # b has ended: c takes its slot
             if fed[r] == 0 and state is not None:
                 state[slot[r], 1] = 0.0  # (the engine zeroes the slots of the requests that start)
+                if pair:
+                    state[slot[r], 0] = 0.0
             rows.append(seqs[r][fed[r]:fed[r] + n])
             starts.append(starts[-1] + n)
             slots.append(slot[r])
         view = None if state is None else state[:, 1]
-        out = ops.causal_conv(torch.cat(rows).cuda(), w.cuda(), view, i32(starts), i32(slots), dtype).float().cpu()
+        if pair:
+            rows0 = torch.cat([seqs0[r][fed[r]:fed[r] + n] for r, n in step]).cuda()
+            out0, out = ops.causal_conv(rows0, w0.cuda(), None if state is None else state[:, 0], i32(starts), i32(slots), dtype,
+                                        torch.cat(rows).cuda(), w.cuda(), view)
+            out0, out = out0.float().cpu(), out.float().cpu()
+        else:
+            out = ops.causal_conv(torch.cat(rows).cuda(), w.cuda(), view, i32(starts), i32(slots), dtype).float().cpu()
         at = 0
         for r, n in step:
             got[r].append(out[at:at + n])
+            if pair:
+                got0[r].append(out0[at:at + n])
             at += n
             fed[r] += n
     for r, x in seqs.items():
         ref = plain.input_convolution(x.double().numpy(), w.double().numpy())
         assert rel(torch.cat(got[r]), ref) <= tol(dtype, 1e-6), r
-    if state is not None:
+        if pair:
+            ref0 = plain.input_convolution(seqs0[r].double().numpy(), w0.double().numpy())
+            assert rel(torch.cat(got0[r]), ref0) <= tol(dtype, 1e-6), r
+    if state is not None and not pair:
         assert bool((state[:, 0] == 77.0).all())  # the other convolution's inputs were left alone
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m, n, k", [(1, 2, 8), (70, 16, 256), (5, 9, 37), (300, 3, 1030)])
+def test_a_few_float32_outputs_a_row(ops, dtype, m, n, k):
+    """The gates' projection: float32 results of a handful of outputs a row, with a bias, at sizes that are multiples
+    of nothing; a row's numbers do not depend on the other rows."""
+    x, w, b = rnd((m, k), 1).to(dtype), rnd((n, k), 2, k ** -0.5).to(dtype), rnd((n,), 3)
+    y = ops.gemm(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, kind=ops.GEMM_NARROW)
+    assert y.dtype == torch.float32
+    ref = x.double().numpy() @ w.double().numpy().T + b.double().numpy()
+    assert rel(y.cpu(), ref) <= 2e-6
+    alone = ops.gemm(x[m // 2:m // 2 + 1].cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, kind=ops.GEMM_NARROW)
+    assert torch.equal(alone[0], y[m // 2])
 
 
 def attention_case(seqs, heads, kv, hd, page, dtype, seed, scalar, edit=None):
