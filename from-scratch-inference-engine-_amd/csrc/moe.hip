@@ -179,6 +179,18 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restri
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
+// Workgroups go to the chip's eight dies in turn, and a die has its own L2.  Die d takes the tiles
+// [d per_die, (d + 1) per_die) of the table (neighbouring tiles are mostly one expert's: a die reads an eighth of the
+// experts' weights, not all of them) and walks them for one block of outputs before it goes to the next block, so
+// that its tiles' rows stay in its L2 meanwhile.
+__device__ __forceinline__ bool die_tile(int max_tiles, int n_blocks, int* tile, int* n_block) {
+    const int per_die = (max_tiles + 7) / 8;
+    const int die = blockIdx.x & 7, mine = blockIdx.x >> 3;
+    *n_block = mine / per_die;
+    *tile = die * per_die + (mine - *n_block * per_die);
+    return *tile < max_tiles && *n_block < n_blocks;
+}
+
 // A workgroup of four waves and a tile of 16 MT slots of one expert.  A wave has MT x NB accumulators of 16 x 16 that
 // share the rows' and the weights' fragments: lane l supplies, for the rows' operand, row l % 16 of each of its MT
 // blocks and the values of K that its lane group (l / 16) owns, and the same of NB weight rows for the other operand;
@@ -191,13 +203,16 @@ template <typename T, int MT, int NB, bool KSPLIT>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, const T* __restrict__ w, void* __restrict__ out,
                                                        const int32_t* __restrict__ tiles, const int32_t* __restrict__ order,
                                                        int gather_div, const float* __restrict__ pair_weight, int N, int K,
-                                                       int epilogue) {
+                                                       int epilogue, int max_tiles) {
     __shared__ float red[KSPLIT ? 3 * MT * NB * 4 * 64 : 1];
-    const int32_t* tl = tiles + 3 * blockIdx.x;
+    int tile, n_block;
+    constexpr int kOutputs = KSPLIT ? 16 * NB : 64 * NB;  // outputs a workgroup
+    if (!die_tile(max_tiles, (N + kOutputs - 1) / kOutputs, &tile, &n_block)) return;
+    const int32_t* tl = tiles + 3 * tile;
     const int expert = tl[0], slot0 = tl[1], n_rows = tl[2];
     if (n_rows <= 0) return;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int n0 = (KSPLIT ? blockIdx.y : blockIdx.y * 4 + wave) * 16 * NB;
+    const int n0 = (KSPLIT ? n_block : n_block * 4 + wave) * 16 * NB;
     if (n0 >= N) return;  // (KSPLIT: the same for the whole workgroup)
     const int r = lane & 15, g = lane >> 4;
     const T* arow[MT];
@@ -385,11 +400,12 @@ extern "C" int fsie_moe_gemm(const void* a, const void* w, void* out, const int3
     FSIE_REQUIRE(epilogue == 0 || (epilogue == 1 && pair_weight), "moe_gemm: unknown epilogue %d", epilogue);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "moe_gemm: unknown dtype %d", dtype);
     if (max_tiles == 0) return 0;
+    const int64_t per_die = ceil_div64(max_tiles, 8);
+    FSIE_REQUIRE(per_die * 8 * ceil_div64(N, 16) <= 0x7fffffff, "moe_gemm: too many tiles");
 #define FSIE_MOE_GEMM(T, MT, NB, KSPLIT)                                                                                 \
-    moe_gemm_kernel<T, MT, NB, KSPLIT><<<dim3(static_cast<unsigned>(max_tiles),                                           \
-                                              static_cast<unsigned>(ceil_div64(N, KSPLIT ? 16 * NB : 64 * NB))),           \
+    moe_gemm_kernel<T, MT, NB, KSPLIT><<<static_cast<unsigned>(per_die * 8 * ceil_div64(N, KSPLIT ? 16 * NB : 64 * NB)),    \
                                          256, 0, stream>>>(static_cast<const T*>(a), static_cast<const T*>(w), out, tiles, order, \
-                                                           gather_div, pair_weight, N, K, epilogue)
+                                                           gather_div, pair_weight, N, K, epilogue, max_tiles)
 #define FSIE_MOE_GEMM_T(T)                                      \
     if (tile_rows == 16) FSIE_MOE_GEMM(T, 1, 2, true);          \
     else if (tile_rows == 64) FSIE_MOE_GEMM(T, 4, 4, false);    \

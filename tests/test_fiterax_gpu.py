@@ -455,10 +455,12 @@ def test_routed_experts_against_the_plain_ones(ops, dtype, t, hidden, ff, expert
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_experts_products_do_not_depend_on_the_tiles(ops, dtype):
+@pytest.mark.parametrize("hidden, ff", [(72, 50), (64, 192), (128, 64)])
+def test_experts_products_do_not_depend_on_the_tiles(ops, dtype, hidden, ff):
     """Tiles of 16, 64 and 128 rows (a few rows an expert, many, very many) over the same pairs: the same products
-    up to the order of their sums, whichever expert is crowded or empty, at sizes that are multiples of nothing."""
-    t, top, n_experts, hidden, ff = 333, 2, 5, 72, 50
+    up to the order of their sums, whichever expert is crowded or empty, at sizes that are multiples of nothing and
+    at sizes that the vector loads take."""
+    t, top, n_experts = 333, 2, 5
     assert [ops.moe_tile_rows(n, 8) for n in (16, 8 * 47, 8 * 48, 8 * 255, 8 * 256)] == [16, 16, 64, 64, 128]
     x = rnd((t, hidden), 1).to(dtype).cuda()
     up = rnd((n_experts, ff, hidden), 2, hidden ** -0.5).to(dtype).cuda()
