@@ -208,7 +208,8 @@ int launch_skinny(const void* x, const void* w, const float* bias, void* y, int 
     return launch_skinny_mt<T, OutT, 8>(x, w, bias, y, M, N, K, stream);
 }
 
-// Few outputs a row (gates, routers): a wave a row of x, float32 results; the matrix stays in cache.
+// Few outputs a row (gates, routers): a wave a row of x and eight outputs (grid.y), float32 results; the matrix stays
+// in cache.
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_narrow_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const float* __restrict__ bias, float* __restrict__ y, int M, int N,
@@ -218,15 +219,14 @@ __global__ __launch_bounds__(256) void gemm_narrow_kernel(const T* __restrict__ 
     if (m >= M) return;
     const T* row = x + static_cast<int64_t>(m) * K;
     const bool vec = wave_dots_vec(x, w, K);
-    for (int n0 = 0; n0 < N; n0 += kWaveDots) {
-        float z[kWaveDots];
-        wave_dots(row, w, K, n0, N, vec, lane, z);
-        float mine = 0.f;
+    const int n0 = blockIdx.y * kWaveDots;
+    float z[kWaveDots];
+    wave_dots(row, w, K, n0, N, vec, lane, z);
+    float mine = 0.f;
 #pragma unroll
-        for (int i = 0; i < kWaveDots; ++i)
-            if (lane == i) mine = z[i];
-        if (lane < kWaveDots && n0 + lane < N) y[static_cast<int64_t>(m) * N + n0 + lane] = mine + (bias ? bias[n0 + lane] : 0.f);
-    }
+    for (int i = 0; i < kWaveDots; ++i)
+        if (lane == i) mine = z[i];
+    if (lane < kWaveDots && n0 + lane < N) y[static_cast<int64_t>(m) * N + n0 + lane] = mine + (bias ? bias[n0 + lane] : 0.f);
 }
 
 }  // namespace
@@ -241,7 +241,8 @@ extern "C" int fsie_gemm(const void* x, const void* w, const float* bias, void* 
     if (kind == 3) {
         FSIE_REQUIRE(out_f32 || dtype == FSIE_F32, "gemm: the narrow kernel writes float32");
         if (M == 0) return 0;
-        const unsigned grid = static_cast<unsigned>((M + 3) / 4);
+        FSIE_REQUIRE(N <= 65535 * kWaveDots, "gemm: %d outputs are too many for the narrow kernel", N);
+        const dim3 grid(static_cast<unsigned>((M + 3) / 4), static_cast<unsigned>((N + kWaveDots - 1) / kWaveDots));
         if (dtype == FSIE_F32)
             gemm_narrow_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x), static_cast<const float*>(w), bias,
                                                                 static_cast<float*>(y), M, N, K);

@@ -207,7 +207,13 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
     __shared__ float red[KSPLIT ? 3 * MT * NB * 4 * 64 : 1];
     int tile, n_block;
     constexpr int kOutputs = KSPLIT ? 16 * NB : 64 * NB;  // outputs a workgroup
-    if (!die_tile(max_tiles, (N + kOutputs - 1) / kOutputs, &tile, &n_block)) return;
+    if constexpr (KSPLIT) {
+        // a handful of tiles, every weight read once: neighbouring workgroups take different tiles, so that every die
+        // has its share of every expert's read
+        tile = blockIdx.x % max_tiles, n_block = blockIdx.x / max_tiles;
+    } else if (!die_tile(max_tiles, (N + kOutputs - 1) / kOutputs, &tile, &n_block)) {
+        return;
+    }
     const int32_t* tl = tiles + 3 * tile;
     const int expert = tl[0], slot0 = tl[1], n_rows = tl[2];
     if (n_rows <= 0) return;
@@ -242,25 +248,33 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
         const bool vec = (K & 7) == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
         union Frag { uint4 raw; bf16x8 v; uint16_t h[8]; };
         if (vec) {
+            // KSPLIT: a wave takes two steps side by side (a whole 128-byte line of every row) of every eight, and
+            // asks for both before it multiplies
+            constexpr int PAIR = KSPLIT ? 2 : 1;
 #pragma unroll 2
-            for (int k0 = KSPLIT ? wave * 32 : 0; k0 < K; k0 += KSPLIT ? 128 : 32) {
-                const int k = k0 + 8 * g;
-                Frag fa[MT], fb[NB];
+            for (int kb = KSPLIT ? wave * 64 : 0; kb < K; kb += KSPLIT ? 256 : 32) {
+                Frag fa[PAIR][MT], fb[PAIR][NB];
 #pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    fa[i].raw = uint4{0, 0, 0, 0};
-                    if (row_in[i] && k < K) fa[i].raw = *reinterpret_cast<const uint4*>(arow[i] + k);
+                for (int st = 0; st < PAIR; ++st) {
+                    const int k = kb + 32 * st + 8 * g;
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        fa[st][i].raw = uint4{0, 0, 0, 0};
+                        if (row_in[i] && k < K) fa[st][i].raw = *reinterpret_cast<const uint4*>(arow[i] + k);
+                    }
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) {
+                        fb[st][j].raw = uint4{0, 0, 0, 0};
+                        if (col_in[j] && k < K) fb[st][j].raw = *reinterpret_cast<const uint4*>(wrow[j] + k);
+                    }
                 }
 #pragma unroll
-                for (int j = 0; j < NB; ++j) {
-                    fb[j].raw = uint4{0, 0, 0, 0};
-                    if (col_in[j] && k < K) fb[j].raw = *reinterpret_cast<const uint4*>(wrow[j] + k);
-                }
+                for (int st = 0; st < PAIR; ++st)
 #pragma unroll
-                for (int i = 0; i < MT; ++i)
+                    for (int i = 0; i < MT; ++i)
 #pragma unroll
-                    for (int j = 0; j < NB; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i].v, fb[j].v, acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < NB; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[st][i].v, fb[st][j].v, acc[i][j], 0, 0, 0);
             }
         } else {
             for (int k0 = KSPLIT ? wave * 32 : 0; k0 < K; k0 += KSPLIT ? 128 : 32) {
@@ -338,14 +352,35 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
     }
 }
 
+// grid = (tokens, blocks of 1024 values); VEC: four values a thread
+template <bool VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, const int32_t* __restrict__ slot_of,
                                                           float* __restrict__ y, int top, int hidden) {
     const int t = blockIdx.x;
-    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
-        float sum = 0.f;
-        for (int c = 0; c < top; ++c) sum += rows[static_cast<int64_t>(slot_of[t * top + c]) * hidden + j];
-        y[static_cast<int64_t>(t) * hidden + j] = sum;
+    int slots[kMaxTop];
+#pragma unroll
+    for (int c = 0; c < kMaxTop; ++c) slots[c] = c < top ? slot_of[t * top + c] : 0;
+    constexpr int V = VEC ? 4 : 1;
+    const int j = (blockIdx.y * 256 + threadIdx.x) * V;
+    if (j >= hidden) return;
+    float sum[V];
+#pragma unroll
+    for (int u = 0; u < V; ++u) sum[u] = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMaxTop; ++c) {
+        if (c < top) {
+            const float* src = rows + static_cast<int64_t>(slots[c]) * hidden + j;
+            if constexpr (VEC) {
+                const float4 v = *reinterpret_cast<const float4*>(src);
+                sum[0] += v.x, sum[1] += v.y, sum[2] += v.z, sum[3] += v.w;
+            } else {
+                sum[0] += src[0];
+            }
+        }
     }
+    float* dst = y + static_cast<int64_t>(t) * hidden + j;
+    if constexpr (VEC) *reinterpret_cast<float4*>(dst) = float4{sum[0], sum[1], sum[2], sum[3]};
+    else dst[0] = sum[0];
 }
 
 }  // namespace
@@ -403,7 +438,8 @@ extern "C" int fsie_moe_gemm(const void* a, const void* w, void* out, const int3
     const int64_t per_die = ceil_div64(max_tiles, 8);
     FSIE_REQUIRE(per_die * 8 * ceil_div64(N, 16) <= 0x7fffffff, "moe_gemm: too many tiles");
 #define FSIE_MOE_GEMM(T, MT, NB, KSPLIT)                                                                                 \
-    moe_gemm_kernel<T, MT, NB, KSPLIT><<<static_cast<unsigned>(per_die * 8 * ceil_div64(N, KSPLIT ? 16 * NB : 64 * NB)),    \
+    moe_gemm_kernel<T, MT, NB, KSPLIT><<<static_cast<unsigned>((KSPLIT ? max_tiles : per_die * 8) *                        \
+                                                               ceil_div64(N, KSPLIT ? 16 * NB : 64 * NB)),                  \
                                          256, 0, stream>>>(static_cast<const T*>(a), static_cast<const T*>(w), out, tiles, order, \
                                                            gather_div, pair_weight, N, K, epilogue, max_tiles)
 #define FSIE_MOE_GEMM_T(T)                                      \
@@ -422,7 +458,11 @@ extern "C" int fsie_moe_combine(const float* rows, const int32_t* slot_of, float
     FSIE_REQUIRE(n_tokens >= 0 && top > 0 && hidden > 0, "moe_combine: bad sizes");
     FSIE_REQUIRE(rows && slot_of && y, "moe_combine: missing operand");
     if (n_tokens == 0) return 0;
-    moe_combine_kernel<<<n_tokens, 256, 0, stream>>>(rows, slot_of, y, top, hidden);
+    FSIE_REQUIRE(top <= kMaxTop, "moe_combine: top %d (at most %d)", top, kMaxTop);
+    const bool vec = hidden % 4 == 0 && (reinterpret_cast<uintptr_t>(rows) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const dim3 grid(n_tokens, static_cast<unsigned>(ceil_div64(hidden, vec ? 1024 : 256)));
+    if (vec) moe_combine_kernel<true><<<grid, 256, 0, stream>>>(rows, slot_of, y, top, hidden);
+    else moe_combine_kernel<false><<<grid, 256, 0, stream>>>(rows, slot_of, y, top, hidden);
     FSIE_CHECK_LAUNCH("moe_combine");
     return 0;
 }
