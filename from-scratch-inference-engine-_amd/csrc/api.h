@@ -297,7 +297,7 @@ int fsie_moe_group(const int32_t* ids, int n_pairs, int experts, int tile_rows, 
                    int32_t* tiles, int max_tiles, hipStream_t stream);
 // One product per expert over its tiles: out[slot] = epilogue(A[row(slot)] . W[expert]^T), W [experts][N][K] in `dtype`.
 // gather_div > 0: row(slot) = order[slot] / gather_div (rows of A are tokens); 0: row(slot) = slot.
-// epilogue 0: exact GELU, out in `dtype`; 1: times slot_weight[order[slot]], out float32.  tile_rows: 16, 64 or 128,
+// epilogue 0: exact GELU, out in `dtype`; 1: times slot_weight[order[slot]], out float32.  tile_rows: 16, 32, 64 or 128,
 // the rows of a tile of `tiles`; fsie_moe_tile_rows names the one that suits a step of n_pairs pairs.
 int fsie_moe_tile_rows(int n_pairs, int experts);
 int fsie_moe_gemm(const void* a, const void* w, void* out, const int32_t* tiles, int max_tiles, const int32_t* order,

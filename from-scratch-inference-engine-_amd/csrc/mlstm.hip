@@ -11,10 +11,11 @@
 //   gates  a wave per (request, head): the activations of 64 tokens at a time, a token a lane, then the running
 //          maximum in the tokens' order (the same few instructions in all lanes); it carries m in the state and
 //          leaves (f, i, m before, m) per token and head
-//   scan   portions below sixteen tokens, single decoded tokens among them: a wave per (request, head, 16 value
-//          columns) walks the tokens in order; lane = (channel quarter, column) holds a quarter of the key channels of
-//          its column of S in registers and the four quarters' shares of S^T q meet through lane exchanges; one more
-//          wave per (request, head) carries n and leaves n . q
+//   scan   portions below sixteen tokens, single decoded tokens among them: a wave per (request, head, 64 value
+//          columns) walks the tokens in order with its columns of S in registers, a column a lane (heads of more
+//          than 128 key channels: two or four lane groups split the channels, 32 or 16 columns a wave, and the
+//          groups' shares of S^T q meet through lane exchanges); one more wave per (request, head) carries n and
+//          leaves n . q
 //   chunks longer portions go sixteen tokens at a time on the matrix cores.  With b_t the sum of f over the chunk's
 //          tokens up to t and m_in the maximum that the chunk starts from,
 //            S_t = exp(b_t + m_in - m_t) S_in + sum_{j <= t} exp(b_t - b_j + i_j - m_t) k_j v_j^T,
@@ -32,8 +33,6 @@
 
 namespace {
 
-constexpr int kCols = 16;        // value columns a wave
-constexpr int kQuarters = 4;     // lane groups that split the key channels
 constexpr int kMaxDim = 512;     // key channels a head
 constexpr int kMaxChunkDim = 256;  // ... of a head whose long portions go chunk by chunk
 constexpr int kPrepThreads = 256;
@@ -177,8 +176,10 @@ __global__ __launch_bounds__(kPrepThreads) void mlstm_chunk_prep_kernel(
     }
 }
 
-// NI: channels a lane holds (its quarter's share, rounded up); channel of register i: i * 4 + quarter
-template <typename T, int NI>
+// Q lane groups split the key channels (one group for heads of up to 128 channels: a wave then reads and writes
+// whole rows of 64 columns of S, 256 bytes side by side); NI: channels a lane holds (its group's share, rounded up);
+// channel of register i: i * Q + group; a wave has 64 / Q value columns.
+template <typename T, int NI, int Q>
 __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ proj, int64_t stride, int q_off, int k_off,
                                                         int v_off, float q_scale, float* __restrict__ state, int64_t record,
                                                         int n_slots, const int32_t* __restrict__ q_starts,
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ pr
     if (rec && last - first >= skip_from) return;  // the chunk kernels' portion
     if (tile == col_tiles) {
         // the normaliser: lane l holds channels l, l + 64, ...
-        constexpr int NN = (NI * kQuarters + 63) / 64;
+        constexpr int NN = (NI * Q + 63) / 64;
         float n[NN];
         float* n_state = rec ? rec + static_cast<int64_t>(dim) * vdim : nullptr;
 #pragma unroll
@@ -228,12 +229,13 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ pr
         }
         return;
     }
-    const int quarter = lane >> 4, col = tile * kCols + (lane & 15);
+    constexpr int COLS = 64 / Q;
+    const int quarter = lane / COLS, col = tile * COLS + lane % COLS;
     const bool col_in = col < vdim;
     float S[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        const int c = i * kQuarters + quarter;
+        const int c = i * Q + quarter;
         S[i] = (rec && col_in && c < dim) ? rec[static_cast<int64_t>(c) * vdim + col] : 0.f;
     }
     for (int t = first; t < last; ++t) {
@@ -244,22 +246,22 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ pr
         float o = 0.f;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int c = i * kQuarters + quarter;
+            const int c = i * Q + quarter;
             const bool in = c < dim;
             const float k = in ? to_float(row[k_off + h * dim + c]) : 0.f;
             const float q = in ? to_float(row[q_off + h * dim + c]) * q_scale : 0.f;
             S[i] = fmaf(cf.x, S[i], k * v);
             o = fmaf(S[i], q, o);
         }
-        // the four quarters' shares, always in the same order
-        o += __shfl_xor(o, 16, FSIE_WAVE);
-        o += __shfl_xor(o, 32, FSIE_WAVE);
+        // the groups' shares, always in the same order
+#pragma unroll
+        for (int off = COLS; off < 64; off <<= 1) o += __shfl_xor(o, off, FSIE_WAVE);
         if (quarter == 0 && col_in) num[(static_cast<int64_t>(t) * heads + h) * vdim + col] = o;
     }
     if (rec && col_in) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int c = i * kQuarters + quarter;
+            const int c = i * Q + quarter;
             if (c < dim) rec[static_cast<int64_t>(c) * vdim + col] = S[i];
         }
     }
@@ -332,7 +334,12 @@ extern "C" int fsie_mlstm_scan(const void* proj, int64_t stride, int q_off, int 
     const int64_t record = fsie_mlstm_state_floats(dim, vdim);
     const int64_t n_at = static_cast<int64_t>(dim) * vdim;
     const int64_t m_at = n_at + dim;
-    const int col_tiles = (vdim + kCols - 1) / kCols;
+    // lane groups of the token-by-token walk: as few as the head's channels allow where that still leaves the chip four
+    // waves a unit (whole rows of S a wave), else four (four times the waves, each with less to wait for)
+    const bool wide = static_cast<int64_t>(n_seqs) * heads * ((vdim + 63) / 64) >= 1024;
+    const int groups = dim > 256 || !wide ? 4 : dim > 128 ? 2 : 1;
+    const int col_tiles = (vdim + 64 / groups - 1) / (64 / groups);
+    const int chunk_tiles = (vdim + 15) / 16;
     FSIE_REQUIRE(heads <= 65535 && col_tiles + 1 <= 65535, "mlstm_scan: too many heads or columns");
     const bool chunks = chunk_work != nullptr && n_tokens >= kGlaChunkMin && dim <= kMaxChunkDim;
     if (chunks) {
@@ -347,28 +354,32 @@ extern "C" int fsie_mlstm_scan(const void* proj, int64_t stride, int q_off, int 
     mlstm_gates_kernel<<<n_seqs * heads, 64, 0, stream>>>(gates, gate_cap, state, record, m_at, n_slots, q_starts, seq_slots,
                                                           heads, coef);
     FSIE_CHECK_LAUNCH("mlstm_gates");
-    const dim3 grid(n_seqs, heads, col_tiles + 1);
-    const int per_lane = (dim + kQuarters - 1) / kQuarters;
+    const dim3 grid(n_seqs, heads, col_tiles + 1), chunk_grid(n_seqs, heads, chunk_tiles + 1);
+    const int per_lane = (dim + groups - 1) / groups;
     int scan_waves = 1;  // a wave for every sixteen key channels, rounded up to a power of two: at most sixteen
     while (scan_waves * 16 < dim) scan_waves *= 2;
     const int dp = 16 * scan_waves;
     const dim3 prep_grid(chunks ? max_chunks : 1, heads);
     const size_t prep_lds = 2 * kGlaChunk * (dp + 4) * sizeof(float);
     const int64_t out_plane = static_cast<int64_t>(n_tokens) * heads * vdim;
-#define FSIE_MLSTM(T, NI)                                                                                              \
-    mlstm_scan_kernel<T, NI><<<grid, 64, 0, stream>>>(static_cast<const T*>(proj), stride, q_off, k_off, v_off, q_scale, state, \
+#define FSIE_MLSTM(T, NI, Q)                                                                                              \
+    mlstm_scan_kernel<T, NI, Q><<<grid, 64, 0, stream>>>(static_cast<const T*>(proj), stride, q_off, k_off, v_off, q_scale, state, \
                                                       record, n_slots, q_starts, seq_slots, heads, dim, vdim, coef, num, den, \
                                                       col_tiles, skip_from)
 #define FSIE_MLSTM_CHUNKS(T, NW)                                                                                       \
-    gla_chunk_scan_kernel<T, NW, true><<<grid, 64 * NW, 0, stream>>>(static_cast<const T*>(proj), stride, v_off, chunk_work,    \
+    gla_chunk_scan_kernel<T, NW, true><<<chunk_grid, 64 * NW, 0, stream>>>(static_cast<const T*>(proj), stride, v_off, chunk_work,    \
                                                                      state, q_starts, seq_slots, num, out_plane, heads, dim,   \
                                                                      vdim, dp, 1, n_slots, record, n_at, den)
 #define FSIE_MLSTM_T(T)                                                                                                \
-    if (per_lane <= 8) FSIE_MLSTM(T, 8);                                                                               \
-    else if (per_lane <= 16) FSIE_MLSTM(T, 16);                                                                        \
-    else if (per_lane <= 32) FSIE_MLSTM(T, 32);                                                                        \
-    else if (per_lane <= 64) FSIE_MLSTM(T, 64);                                                                        \
-    else FSIE_MLSTM(T, 128);                                                                                           \
+    if (groups == 4 && per_lane <= 8) FSIE_MLSTM(T, 8, 4);                                                             \
+    else if (groups == 4 && per_lane <= 16) FSIE_MLSTM(T, 16, 4);                                                      \
+    else if (groups == 4 && per_lane <= 32) FSIE_MLSTM(T, 32, 4);                                                      \
+    else if (groups == 4 && per_lane <= 64) FSIE_MLSTM(T, 64, 4);                                                      \
+    else if (groups == 4) FSIE_MLSTM(T, 128, 4);                                                                       \
+    else if (groups == 2) FSIE_MLSTM(T, 128, 2);                                                                       \
+    else if (per_lane <= 32) FSIE_MLSTM(T, 32, 1);                                                                     \
+    else if (per_lane <= 64) FSIE_MLSTM(T, 64, 1);                                                                     \
+    else FSIE_MLSTM(T, 128, 1);                                                                                        \
     if (chunks) {                                                                                                      \
         mlstm_chunk_prep_kernel<T><<<prep_grid, kPrepThreads, prep_lds, stream>>>(                                      \
             static_cast<const T*>(proj), stride, q_off, k_off, coef, chunk_work, q_starts, seq_slots, n_seqs, heads, dim, dp,   \

@@ -5,7 +5,7 @@
 //            score + correction (ties to the lower index), weights = chosen scores / their sum * scale
 //   group    one workgroup: counts per expert, starts, a slot for every pair (pairs of one expert keep the order
 //            of the pairs), and the table of row tiles (expert, first slot, slots) that never cross an expert
-//   gemm     a workgroup per tile of 16, 64 or 128 slots of one expert on the matrix cores: bfloat16 operands
+//   gemm     a workgroup per tile of 16, 32, 64 or 128 slots of one expert on the matrix cores: bfloat16 operands
 //            (mfma 16x16x32) or true float32 ones (mfma 16x16x4); both operands run along K in memory, which is
 //            the order the instruction wants; rows are gathered through the order table; the epilogue is the exact
 //            GELU (up) or the pair's routing weight (down, float32 result)
@@ -418,19 +418,20 @@ extern "C" int fsie_moe_group(const int32_t* ids, int n_pairs, int experts, int 
 }
 
 // Rows of a tile that the products are best run with for this many (token, choice) pairs over this many experts: 16
-// (the weights' read bounds the product: the waves split K), 64 or 128 (a weight fragment serves four or eight
-// blocks of rows).  fsie_moe_group and fsie_moe_gemm take any of the three.
+// or 32 (the weights' read bounds the product: the waves split K, and an expert's rows should fit one tile so that
+// its weights are read once), 64 or 128 (a weight fragment serves four or eight blocks of rows).  fsie_moe_group and
+// fsie_moe_gemm take any of the four.
 extern "C" int fsie_moe_tile_rows(int n_pairs, int experts) {
     const int per_expert = n_pairs / (experts > 0 ? experts : 1);
-    return per_expert >= 256 ? 128 : per_expert >= 48 ? 64 : 16;
+    return per_expert >= 256 ? 128 : per_expert >= 48 ? 64 : per_expert > 8 ? 32 : 16;
 }
 
 extern "C" int fsie_moe_gemm(const void* a, const void* w, void* out, const int32_t* tiles, int max_tiles,
                              const int32_t* order, int gather_div, const float* pair_weight, int N, int K, int epilogue,
                              int dtype, int tile_rows, hipStream_t stream) {
     FSIE_REQUIRE(max_tiles >= 0 && N > 0 && K > 0 && gather_div >= 0, "moe_gemm: bad sizes tiles=%d N=%d K=%d", max_tiles, N, K);
-    FSIE_REQUIRE(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_gemm: tiles of %d rows (the kernels take 16, 64, 128)",
-                 tile_rows);
+    FSIE_REQUIRE(tile_rows == 16 || tile_rows == 32 || tile_rows == 64 || tile_rows == 128,
+                 "moe_gemm: tiles of %d rows (the kernels take 16, 32, 64, 128)", tile_rows);
     FSIE_REQUIRE(a && w && out && tiles && order, "moe_gemm: missing operand");
     FSIE_REQUIRE(epilogue == 0 || (epilogue == 1 && pair_weight), "moe_gemm: unknown epilogue %d", epilogue);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "moe_gemm: unknown dtype %d", dtype);
@@ -444,6 +445,7 @@ extern "C" int fsie_moe_gemm(const void* a, const void* w, void* out, const int3
                                                            gather_div, pair_weight, N, K, epilogue, max_tiles)
 #define FSIE_MOE_GEMM_T(T)                                      \
     if (tile_rows == 16) FSIE_MOE_GEMM(T, 1, 2, true);          \
+    else if (tile_rows == 32) FSIE_MOE_GEMM(T, 2, 2, true);     \
     else if (tile_rows == 64) FSIE_MOE_GEMM(T, 4, 4, false);    \
     else FSIE_MOE_GEMM(T, 8, 4, false)
     if (dtype == FSIE_F32) { FSIE_MOE_GEMM_T(float); } else { FSIE_MOE_GEMM_T(bf16_t); }

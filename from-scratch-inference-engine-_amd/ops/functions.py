@@ -1164,7 +1164,7 @@ def mlstm_out(num: torch.Tensor, den: torch.Tensor, coef: torch.Tensor, gate: to
 
 
 def moe_tile_rows(n_pairs: int, experts: int) -> int:
-    """Rows of a tile of the experts' products for a step of this many (token, choice) pairs: 16, 64 or 128."""
+    """Rows of a tile of the experts' products for a step of this many (token, choice) pairs: 16, 32, 64 or 128."""
     return int(load().fsie_moe_tile_rows(int(n_pairs), int(experts)))
 
 

@@ -347,7 +347,8 @@ def oracle_memory(proj, gates, heads, dim, vdim, cap, pieces=False):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads, dim, vdim, cap", [(4, 32, 48, 12.0), (1, 20, 7, 3.0), (3, 130, 33, 15.0), (2, 256, 64, 8.0)])
+@pytest.mark.parametrize("heads, dim, vdim, cap", [(4, 32, 48, 12.0), (1, 20, 7, 3.0), (3, 130, 33, 15.0), (2, 256, 64, 8.0),
+                                                   (1, 300, 70, 5.0)])
 def test_matrix_memory_over_portions_steps_and_slots(ops, dtype, heads, dim, vdim, cap):
     """Requests fed whole, token by token and in unequal portions, in slots that are used again: numerator, the
     normaliser's product and the running maximum of every token are those of the walk over the whole request, with
@@ -398,6 +399,31 @@ def test_matrix_memory_over_portions_steps_and_slots(ops, dtype, heads, dim, vdi
         mine = ref["a"][0]
         assert np.abs(other[-1, 1] - mine[-1, 1]).max() > 0.05 * np.abs(mine[-1, 1]).max()
         assert np.abs(other[-1, 0] - mine[-1, 0]).max() < 1e-6 * np.abs(mine[-1, 0]).max()
+
+
+@pytest.mark.parametrize("dim, vdim", [(24, 40), (140, 20), (64, 100)])
+def test_matrix_memory_of_many_requests_a_step(ops, dim, vdim):
+    """Steps of 128 requests (two tokens each, then single tokens): with that many the walk holds whole rows of the
+    memory a wave; the same numbers as with a few requests, against the plain walk."""
+    n, heads, cap, dtype = 128, 8, 9.0, torch.float32
+    data = [memory_inputs(5, heads, dim, vdim, 7 * r, dtype) for r in range(n)]
+    state = torch.zeros((n, heads, ops.mlstm_state_floats(dim, vdim))).cuda()
+    got = [[] for _ in range(n)]
+    fed = 0
+    for size in (2, 1, 1, 1):
+        proj = torch.cat([p[fed:fed + size] for p, _ in data]).cuda()
+        gates = torch.cat([g[fed:fed + size] for _, g in data]).cuda()
+        num, den, coef = ops.mlstm_scan(proj, 0, heads * dim, 2 * heads * dim, gates, cap, dim ** -0.5, state,
+                                        i32(list(range(0, n * size + 1, size))), i32(list(range(n))), heads, dim, vdim)
+        num, den = num.cpu(), den.cpu()
+        for r in range(n):
+            got[r].append((num[r * size:(r + 1) * size], den[r * size:(r + 1) * size]))
+        fed += size
+    for r in range(0, n, 9):
+        _, ref_num, ref_den, _ = oracle_memory(*data[r], heads, dim, vdim, cap, pieces=True)
+        num, den = (torch.cat([g[i] for g in got[r]]).numpy() for i in range(2))
+        for h in range(heads):
+            assert rel(num[:, h], ref_num[:, h]) <= 2e-5 and rel(den[:, h], ref_den[:, h]) <= 2e-5, (r, h)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -457,11 +483,11 @@ def test_routed_experts_against_the_plain_ones(ops, dtype, t, hidden, ff, expert
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hidden, ff", [(72, 50), (64, 192), (128, 64)])
 def test_experts_products_do_not_depend_on_the_tiles(ops, dtype, hidden, ff):
-    """Tiles of 16, 64 and 128 rows (a few rows an expert, many, very many) over the same pairs: the same products
+    """Tiles of 16, 32, 64 and 128 rows (a few rows an expert, many, very many) over the same pairs: the same products
     up to the order of their sums, whichever expert is crowded or empty, at sizes that are multiples of nothing and
     at sizes that the vector loads take."""
     t, top, n_experts = 333, 2, 5
-    assert [ops.moe_tile_rows(n, 8) for n in (16, 8 * 47, 8 * 48, 8 * 255, 8 * 256)] == [16, 16, 64, 64, 128]
+    assert [ops.moe_tile_rows(n, 8) for n in (16, 8 * 8, 8 * 9, 8 * 47, 8 * 48, 8 * 255, 8 * 256)] == [16, 16, 32, 32, 64, 64, 128]
     x = rnd((t, hidden), 1).to(dtype).cuda()
     up = rnd((n_experts, ff, hidden), 2, hidden ** -0.5).to(dtype).cuda()
     down = rnd((n_experts, hidden, ff), 3, ff ** -0.5).to(dtype).cuda()
@@ -469,7 +495,7 @@ def test_experts_products_do_not_depend_on_the_tiles(ops, dtype, hidden, ff):
     ids[:200, 0] = 1  # a crowded one
     weights = rnd((t * top,), 5).abs().cuda()
     got = {}
-    for rows in (16, 64, 128):
+    for rows in (16, 32, 64, 128):
         order, slot_of, tiles = ops.moe_group(ids.cuda(), n_experts, tile_rows=rows)
         act = ops.moe_gemm(x, up, tiles, order, gather_div=top, tile_rows=rows)
         out = ops.moe_gemm(act, down, tiles, order, pair_weight=weights, tile_rows=rows)
@@ -482,7 +508,7 @@ def test_experts_products_do_not_depend_on_the_tiles(ops, dtype, hidden, ff):
             if dtype == torch.bfloat16:
                 hid = torch.tensor(hid).to(dtype).double().numpy()
             ref[i] += float(weights[i * top + c]) * (down[e[i, c]].cpu().double().numpy() @ hid)
-    for rows in (16, 64, 128):
+    for rows in (16, 32, 64, 128):
         assert rel(got[rows], ref) <= tol(dtype, 2e-5, 2.0 ** -6), rows
         assert rel(got[rows], got[16]) <= tol(dtype, 2e-6, 2.0 ** -7), rows
 
