@@ -275,13 +275,13 @@ def fiterax_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
     the experts together hold as many weights as the dense feed-forward of the same ``ff``."""
     heads = width // 128
     memory = {"heads": width // 256, "dim": 128, "vdim": 256, "gate_cap": 15.0}
-    gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
+    gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
            "rot": {"base": 500000.0, "dims": 64}}
-    mlp = {"kind": "moe", "expert": {"ff": ff * 3 // 16}, "router": {"experts": 8, "top": 2, "scale": 2.5}}
+    mlp = {"kind": "moe", "expert": {"ff": ff * 3 // 16}, "router": {"experts": 8, "top": 2, "scale": 2.0}}
     out = [{"type": "mlstm" if i % 2 == 0 else "attention", "mixer": dict(memory if i % 2 == 0 else gqa), "mlp": dict(mlp)}
            for i in range(layers)]
-    return {"architecture": "Fiterax", "width": width, "vocab": vocab, "norm": {"eps": 1e-5, "groups": 2},
-            "embedding": {"scale": 12.0}, "residual_mult": 0.3, "canon": {"taps": 4}, "layers": out}
+    return {"architecture": "Fiterax", "width": width, "vocab": vocab, "norm": {"eps": 1e-5, "groups": 4},
+            "embedding": {"scale": 10.0}, "residual_mult": 0.25, "canon": {"taps": 4}, "layers": out}
 
 
 DESIGN_SHAPES = {"gilozen": gilozen_shape, "botulorn": botulorn_shape, "fiterax": fiterax_shape}

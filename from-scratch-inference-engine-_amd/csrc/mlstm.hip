@@ -244,14 +244,35 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const T* __restrict__ pr
             const float2 cf = {expf(gm.x + gm.z - gm.w), expf(gm.y - gm.w)};  // keep, take
         const float v = col_in ? to_float(row[v_off + h * vdim + col]) * cf.y : 0.f;  // take * v
         float o = 0.f;
+        if constexpr (Q == 1) {
+            // every lane needs every channel's k and q: a lane reads the channels lane, lane + 64, and each is handed
+            // round from its lane
+            constexpr int NR = (NI + 63) / 64;
+            float kk[NR], qq[NR];
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int c = i * Q + quarter;
-            const bool in = c < dim;
-            const float k = in ? to_float(row[k_off + h * dim + c]) : 0.f;
-            const float q = in ? to_float(row[q_off + h * dim + c]) * q_scale : 0.f;
-            S[i] = fmaf(cf.x, S[i], k * v);
-            o = fmaf(S[i], q, o);
+            for (int j = 0; j < NR; ++j) {
+                const int c = j * 64 + lane;
+                const bool in = c < dim;
+                kk[j] = in ? to_float(row[k_off + h * dim + c]) : 0.f;
+                qq[j] = in ? to_float(row[q_off + h * dim + c]) * q_scale : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const float k = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, kk[i / 64]), i % 64));
+                const float q = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, qq[i / 64]), i % 64));
+                S[i] = fmaf(cf.x, S[i], k * v);
+                o = fmaf(S[i], q, o);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int c = i * Q + quarter;
+                const bool in = c < dim;
+                const float k = in ? to_float(row[k_off + h * dim + c]) : 0.f;
+                const float q = in ? to_float(row[q_off + h * dim + c]) * q_scale : 0.f;
+                S[i] = fmaf(cf.x, S[i], k * v);
+                o = fmaf(S[i], q, o);
+            }
         }
         // the groups' shares, always in the same order
 #pragma unroll
