@@ -97,6 +97,9 @@ int fsie_head_gemm(const void* x, int64_t x_stride, int x_off, int x_hs, const v
                    int y_hs, const float* gate, int n_tokens, int heads, int N, int K, int dtype, hipStream_t stream);
 int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
 int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);
+// y [rows][cols] bfloat16 = parts[0] + parts[1] + ... (float32 [planes][rows][cols], added in their order) + bias
+// (float32 [cols] or null), rounded once; cols a multiple of 4
+int fsie_sum_round(const float* parts, int planes, const float* bias, void* y, int rows, int cols, hipStream_t stream);
 
 int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int32_t* slots, const double* inv_freq,
                        const float* bias, void* k_pool, void* v_pool, int n_tokens, int n_heads, int n_kv, int head_dim,

@@ -293,6 +293,26 @@ __global__ void bias_add_kernel(T* __restrict__ y, const float* __restrict__ bia
     if (i < total) y[i] = from_float<T>(to_float(y[i]) + bias[i % cols]);
 }
 
+// y = sum of `planes` float32 partial sums, added in their order, + bias, rounded once; four values a thread
+__global__ void sum_round_kernel(const float* __restrict__ parts, int planes, int64_t plane, const float* __restrict__ bias,
+                                 bf16_t* __restrict__ y, int64_t total, int cols) {
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+    if (i >= total) return;
+    float4 sum = *reinterpret_cast<const float4*>(parts + i);
+    for (int p = 1; p < planes; ++p) {
+        const float4 v = *reinterpret_cast<const float4*>(parts + p * plane + i);
+        sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+    }
+    if (bias) {
+        const float4 b = *reinterpret_cast<const float4*>(bias + i % cols);
+        sum.x += b.x, sum.y += b.y, sum.z += b.z, sum.w += b.w;
+    }
+    uint2 raw;
+    raw.x = static_cast<uint32_t>(from_float<bf16_t>(sum.x).bits) | static_cast<uint32_t>(from_float<bf16_t>(sum.y).bits) << 16;
+    raw.y = static_cast<uint32_t>(from_float<bf16_t>(sum.z).bits) | static_cast<uint32_t>(from_float<bf16_t>(sum.w).bits) << 16;
+    *reinterpret_cast<uint2*>(y + i) = raw;
+}
+
 // Rows of a table set to zero: row slots[i] of [n_slots, row_bytes / 4] words, negative = none.
 __global__ void zero_rows_kernel(uint32_t* __restrict__ table, const int32_t* __restrict__ slots, int64_t row_words,
                                  int n_slots) {
@@ -529,6 +549,20 @@ extern "C" int fsie_residual_add(float* residual, const void* delta, int64_t tot
         residual_add_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(residual, static_cast<const bf16_t*>(delta), total);
     }
     FSIE_CHECK_LAUNCH("residual_add");
+    return 0;
+}
+
+extern "C" int fsie_sum_round(const float* parts, int planes, const float* bias, void* y, int rows, int cols,
+                              hipStream_t stream) {
+    FSIE_REQUIRE(rows >= 0 && cols > 0 && cols % 4 == 0 && planes >= 1, "sum_round: bad sizes %d x %d, %d planes", rows, cols, planes);
+    FSIE_REQUIRE(parts && y, "sum_round: missing operand");
+    FSIE_REQUIRE((reinterpret_cast<uintptr_t>(parts) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(y) & 7) == 0, "sum_round: operands must be 16-byte aligned");
+    const int64_t total = static_cast<int64_t>(rows) * cols;
+    if (total == 0) return 0;
+    sum_round_kernel<<<static_cast<unsigned>(ceil_div64(total / 4, kThreads)), kThreads, 0, stream>>>(
+        parts, planes, total, bias, static_cast<bf16_t*>(y), total, cols);
+    FSIE_CHECK_LAUNCH("sum_round");
     return 0;
 }
 

@@ -202,6 +202,22 @@ def bias_add(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     return y
 
 
+def sum_round(parts: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bfloat16 [M, N] from float32 partial sums [S, M, N] (or one plane [M, N]): added in their order, plus ``bias``
+    (float32 [N]), rounded once.  N a multiple of 4."""
+    if parts.ndim == 2:
+        parts = parts.unsqueeze(0)
+    _need(parts, "sum_round parts", dtype=torch.float32, ndim=3)
+    s, m, n = parts.shape
+    if n % 4:
+        raise KernelError(f"sum_round: rows of {n} values are not a multiple of four")
+    if bias is not None:
+        _need(bias, "sum_round bias", dtype=torch.float32, shape=(n,))
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=parts.device)
+    check(load().fsie_sum_round(parts.data_ptr(), s, _ptr(bias), y.data_ptr(), m, n, _stream()))
+    return y
+
+
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
                   inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor] = None,
                   k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,

@@ -35,6 +35,7 @@ _SIGNATURES = {
     "fsie_swiglu": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_residual_add": ([_P, _P, c_int64, c_int, _P], c_int),
     "fsie_bias_add": ([_P, _P, c_int, c_int, c_int, _P], c_int),
+    "fsie_sum_round": ([_P, c_int, _P, _P, c_int, c_int, _P], c_int),
     "fsie_rope_kv_write": ([_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
                             c_int, _P], c_int),
     "fsie_rope_kv_write_table": ([_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P, c_int, _P],

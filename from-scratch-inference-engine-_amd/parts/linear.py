@@ -111,6 +111,13 @@ class Linear:
             return library_mm(x, w, float32_result=True)
         if self.in_features % 8 == 0 and m <= (GEMM_MFMA_SKINNY_MAX_M if wants_f32 else GEMM_MFMA_SKINNY_BEST_M):
             return ops.gemm_mfma_skinny(x, w, bias, out_dtype=out_dtype)
+        if not wants_f32 and self.out_features % 4 == 0:
+            # 17 to 64 rows (to 128 from a fragment-ordered copy): the engine's product that shares x through LDS, as
+            # float32 partial sums of slices of K, added up and rounded once; the library needs 40 us for 64 rows of
+            # a matrix whose read is 8 us
+            sums = self.partial_sums(x)
+            if sums is not None:
+                return ops.sum_round(sums, bias)
         if m <= GEMM_SKINNY_MAX_M or wants_f32 or self.in_features % 8 or self.out_features % 8:
             # few rows with an odd inner size; float32 results from bfloat16 operands (logits of
             # many rows); and sizes whose rows are not 16-byte aligned, which the library is not given

@@ -156,6 +156,35 @@ def test_a_few_float32_outputs_a_row(ops, dtype, m, n, k):
     assert torch.equal(alone[0], y[m // 2])
 
 
+@pytest.mark.parametrize("planes, m, n, with_bias", [(1, 3, 8, False), (4, 37, 100, True), (9, 64, 6144, True)])
+def test_partial_sums_added_in_order_and_rounded_once(ops, planes, m, n, with_bias):
+    parts, bias = rnd((planes, m, n), 1, 3.0), rnd((n,), 2)
+    y = ops.sum_round(parts.cuda(), bias.cuda() if with_bias else None)
+    ref = parts[0].clone()
+    for p in range(1, planes):
+        ref += parts[p]
+    if with_bias:
+        ref += bias
+    assert y.dtype == torch.bfloat16 and torch.equal(y.cpu(), ref.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("m", [17, 40, 64])
+def test_products_of_a_few_dozen_rows_from_the_engine(ops, m):
+    """17 to 64 rows with a bfloat16 result: partial sums of the engine's product, added and rounded once, against
+    float64; a row's numbers do not depend on the other rows."""
+    from from_scratch_inference_engine_amd.parts.linear import Linear
+
+    lin = Linear(512, 1544, bias=True)
+    lin.weight, lin.bias = rnd((1544, 512), 1, 512 ** -0.5).to(torch.bfloat16).cuda(), rnd((1544,), 2).cuda()
+    lin.prepare(True)
+    x = rnd((m, 512), 3).to(torch.bfloat16)
+    y = lin(x.cuda())
+    ref = x.double().numpy() @ lin.weight.cpu().double().numpy().T + lin.bias.cpu().double().numpy()
+    assert y.dtype == torch.bfloat16 and rel(y.float().cpu(), ref) <= 2.0 ** -7
+    fewer = lin(x[:m - 7].cuda())
+    assert rel(fewer.float().cpu(), y[:m - 7].float().cpu()) <= 2.0 ** -7
+
+
 def attention_case(seqs, heads, kv, hd, page, dtype, seed, scalar, edit=None):
     """Pools, tables and the planner's items for requests (past, new) of a causal attention without a window."""
     from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
