@@ -66,9 +66,18 @@ __global__ __launch_bounds__(64) void mlstm_gates_kernel(const float* __restrict
             f = log_sigmoid(cap * tanhf(gf / cap));
         }
         float before = 0.f, mine = 0.f;
+        if (nt == 64) {
+            // a full round: nothing but the chain's add and maximum between two tokens
 #pragma unroll
-        for (int j = 0; j < 64; ++j) {
-            if (j < nt) {
+            for (int j = 0; j < 64; ++j) {
+                const float fj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f), j));
+                const float ij = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, i), j));
+                const float m_new = fmaxf(fj + m, ij);
+                if (lane == j) before = m, mine = m_new;
+                m = m_new;
+            }
+        } else {
+            for (int j = 0; j < nt; ++j) {
                 const float fj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f), j));
                 const float ij = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, i), j));
                 const float m_new = fmaxf(fj + m, ij);
