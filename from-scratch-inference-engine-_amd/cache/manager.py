@@ -15,7 +15,7 @@ from dataclasses import dataclass, field
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence, Tuple
 
 from .allocator import OutOfPages, PageAllocator
-from .needs import CacheNeed, PagedNeed, StateNeed  # noqa: F401  (PagedNeed and StateNeed are also named from here)
+from .needs import CacheNeed, PagedNeed, PooledNeed, StateNeed  # noqa: F401  (the needs are also named from here)
 
 
 class NoFreeSlot(RuntimeError):

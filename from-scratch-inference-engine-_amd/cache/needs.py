@@ -146,6 +146,23 @@ class PagedNeed(CacheNeed):
 
 
 @dataclass(frozen=True)
+class PooledNeed(PagedNeed):
+    """One entry per block of ``tokens_per_entry`` consecutive positions and layer: a key and a value for the block as
+    a whole (their means), in pools laid out like those of keys and values.  A group of its own, with its own pages
+    and block tables; the step's slot table names for every token the entry of its block."""
+
+    tokens_per_entry: int = 1
+
+    def __post_init__(self):
+        PagedNeed.__post_init__(self)
+        if self.tokens_per_entry < 1:
+            raise ValueError("PooledNeed: a block holds at least one position")
+
+    def bytes_per_token(self, dtype) -> int:
+        return -(-PagedNeed.bytes_per_token(self, dtype) // self.tokens_per_entry)
+
+
+@dataclass(frozen=True)
 class StateNeed(CacheNeed):
     """A tensor of fixed ``shape`` per request and layer (torch dtype name, e.g. 'float32')."""
 

@@ -28,6 +28,9 @@
 // FSIE_ATTN_KEEP_WALK set the item also reads the keys [0, min(KEEP, KBEGIN)), before those of its own range.
 #define FSIE_ATTN_ITEM_KEEP 7
 #define FSIE_ATTN_KEEP_WALK (1 << 30)
+// with FSIE_ATTN_POOL_WALK set (kernels that take pooled blocks) the item also reads the mean keys and values of the
+// blocks of positions that lie wholly before its queries' windows, from the pools of pooled blocks
+#define FSIE_ATTN_POOL_WALK (1 << 29)
 // one merge item = 4 int32: {output row, first partial slot, number of splits, slot stride}
 #define FSIE_ATTN_MERGE_INTS 4
 
@@ -81,7 +84,9 @@ int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_floats_per_token
 int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* z, float* state,
                   const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, float* prep, float* out,
                   float* chunk_work, int max_chunks, int heads, int dim, int vdim, float q_scale, float inv_tau,
-                  int n_slots, int dtype, hipStream_t stream);
+                  int n_slots, int dtype, const float* head_decay, hipStream_t stream);
+// head_decay (or null): float32 [heads]; with it z may be null and every key channel of head h decays by head_decay[h],
+// the same for every token (retention: a fixed decay a head).
 
 // Attention through a latent (latent_attention.hip): the norms of the latents, the gates and the cache row of
 // every token; the rotation of pairs of neighbours; a product with a matrix of its own for every head.
@@ -95,6 +100,10 @@ int fsie_rope_pairs(const void* in, int64_t in_stride, int in_off, int in_hs, vo
                     int dtype, hipStream_t stream);
 int fsie_head_gemm(const void* x, int64_t x_stride, int x_off, int x_hs, const void* w, void* y, int64_t y_stride, int y_off,
                    int y_hs, const float* gate, int n_tokens, int heads, int N, int K, int dtype, hipStream_t stream);
+// y = x rounded to `dtype` (a copy for float32)
+int fsie_round_to(const float* x, void* y, int64_t total, int dtype, hipStream_t stream);
+// y = a * x1 + b * x2, elementwise, float32 arithmetic, all three of `dtype`
+int fsie_scaled_sum(const void* x1, float a, const void* x2, float b, void* y, int64_t total, int dtype, hipStream_t stream);
 int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
 int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);
 // y [rows][cols] bfloat16 = parts[0] + parts[1] + ... (float32 [planes][rows][cols], added in their order) + bias
@@ -138,7 +147,8 @@ int fsie_attention_prep(const void* proj, int64_t stride, int q_off, int k_off, 
                         int kv_heads, int dim, int vdim, int D, const float* q_weight, const float* k_weight, float eps,
                         int pairs, const float* cos_sin, const void* v_other, int64_t v_other_stride, const float* mix,
                         void* q_out, float* gate, const int32_t* slots, void* k_pool, void* v_pool, int page_size,
-                        int64_t pool_slots, int n_tokens, int dtype, int q_weight_stride, hipStream_t stream);
+                        int64_t pool_slots, int n_tokens, int dtype, int q_weight_stride, int v_unit_norm, float v_eps,
+                        hipStream_t stream);
 int fsie_gate_heads(const void* x, int D, const float* gate, void* y, int n_tokens, int heads, int vdim, int dtype,
                     hipStream_t stream);
 
@@ -182,7 +192,13 @@ int fsie_fragment_order(const void* w, void* out, int N, int K, hipStream_t stre
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
                           void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,
-                          int window, float scale, int dtype, const float* sinks, float softcap, hipStream_t stream);
+                          int window, float scale, int dtype, const float* sinks, float softcap, const void* k_pooled,
+                          const void* v_pooled, const int32_t* pooled_tables, int pooled_max_pages, int pooled_page_size,
+                          int pooled_tokens, hipStream_t stream);
+// k_pooled .. pooled_tokens (or null and zeros): pools [units][n_kv][pooled_page_size][head_dim] and
+// [units][n_kv][head_dim][pooled_page_size] that hold one mean key and value for every block of pooled_tokens positions,
+// with their block table [requests][pooled_max_pages]; an item flagged FSIE_ATTN_POOL_WALK reads, beside its own keys,
+// the blocks that lie wholly before a query's window (fsie_pool_blocks fills them).
 // softcap (in every attention entry point that takes it): a positive number caps the scaled scores,
 // s <- softcap * tanh(s / softcap), before the mask and the softmax; 0: scores as they are.
 // sinks (or null, in every attention entry point that takes it): float32 [n_heads]; exp(sinks[h]) is one more
@@ -191,6 +207,13 @@ int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, c
 int fsie_attention_merge(const float* partials, const int32_t* merges, int n_merges, void* out, int n_heads,
                          int head_dim, int dtype, const float* sinks, hipStream_t stream);
 int fsie_attention_scalar_tile_tokens(int n_heads, int n_kv);
+// The mean key and value of blocks of `block_tokens` consecutive positions, from the pages of keys and values to the
+// pools of pooled blocks: jobs [n_jobs][2] = (request of the step, block), a request of -1: nothing.  Block b's
+// positions b * block_tokens .. are read through the request's row of block_tables and summed in their order in float32;
+// the entry goes to the page that pooled_tables names for b.
+int fsie_pool_blocks(const void* k_pool, const void* v_pool, const int32_t* block_tables, int max_pages, int page_size,
+                     void* k_pooled, void* v_pooled, const int32_t* pooled_tables, int pooled_max_pages, int pooled_page_size,
+                     const int32_t* jobs, int n_jobs, int block_tokens, int n_kv, int head_dim, int dtype, hipStream_t stream);
 
 int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                         const int32_t* block_tables, int max_pages, const int32_t* items, int n_items, void* out,
@@ -292,7 +315,11 @@ int fsie_mlstm_out(const float* num, const float* den, const float* coef, const 
 // `top` experts with the largest s + correction (ties: the lower index) are chosen; their weights are their s divided
 // by the sum of the chosen s (+ 1e-20) times `scale`.  ids [n_tokens][top] int32, weights [n_tokens][top] float32.
 int fsie_moe_route(const void* x, const void* router, const float* correction, int dtype, int32_t* ids, float* weights,
-                   int n_tokens, int hidden, int experts, int top, float scale, hipStream_t stream);
+                   int n_tokens, int hidden, int experts, int top, float scale, int kind, int groups, int keep, int renorm,
+                   hipStream_t stream);
+// kind 0: sigmoid scores, 1: softmax over all experts.  groups > 1: experts in that many equal groups of neighbours, only
+// those of the `keep` groups with the largest best score (+ correction) can be chosen.  renorm 0: the weights are the
+// chosen scores themselves (times scale).  correction may be null.
 // Groups the n = n_tokens * top (token, choice) pairs by expert: order[slot] = pair (slots of one expert are
 // consecutive), slot_of[pair] = slot, and a table of row tiles of `tile_rows` slots that never cross an expert:
 // tiles [max_tiles][3] = (expert, first slot, slots), max_tiles = ceil(n / tile_rows) + experts; unused tiles have 0 slots.
@@ -300,7 +327,8 @@ int fsie_moe_group(const int32_t* ids, int n_pairs, int experts, int tile_rows, 
                    int32_t* tiles, int max_tiles, hipStream_t stream);
 // One product per expert over its tiles: out[slot] = epilogue(A[row(slot)] . W[expert]^T), W [experts][N][K] in `dtype`.
 // gather_div > 0: row(slot) = order[slot] / gather_div (rows of A are tokens); 0: row(slot) = slot.
-// epilogue 0: exact GELU, out in `dtype`; 1: times slot_weight[order[slot]], out float32.  tile_rows: 16, 32, 64 or 128,
+// epilogue 0: exact GELU, out in `dtype`; 1: times slot_weight[order[slot]], out float32; 2 + a (a: FsieGateAct): the rows
+// of W[expert] are gate and up in turn (N even) and out [slots][N / 2] = act(gate) * up in `dtype`.  tile_rows: 16, 32, 64 or 128,
 // the rows of a tile of `tiles`; fsie_moe_tile_rows names the one that suits a step of n_pairs pairs.
 int fsie_moe_tile_rows(int n_pairs, int experts);
 int fsie_moe_gemm(const void* a, const void* w, void* out, const int32_t* tiles, int max_tiles, const int32_t* order,

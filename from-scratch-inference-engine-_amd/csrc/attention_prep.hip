@@ -7,7 +7,8 @@
 //               weights may also differ: head h then takes q_weight + h * q_weight_stride), then the
 //               first 2 * pairs values turned, value i with value i + pairs, by the step's cosines and sines
 //               cos_sin [tokens][pairs][2]; all of it float32
-//   v:          (1 - mix) v + mix * v_other where another layer's values of the same token are given
+//   v:          (1 - mix) v + mix * v_other where another layer's values of the same token are given; with v_unit_norm
+//               every head's values are then divided by sqrt(mean(v^2) + v_eps)
 //   gate:       sigmoid of the logits, float32 [tokens][heads]
 // q goes to q_out [tokens][heads * D] and k, v into the pools at slots[t], heads of D >= max(dim, vdim) values,
 // zeros behind the dim (or vdim) that are used: the attention kernels take one head size for keys and values.
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
     const float2* __restrict__ cos_sin, const T* __restrict__ v_other, int64_t v_other_stride, const float* __restrict__ mix,
     T* __restrict__ q_out, float* __restrict__ gate, const int32_t* __restrict__ slots, T* __restrict__ k_pool,
     T* __restrict__ v_pool, int page_size, int64_t pool_slots, int values_elsewhere, int L, int head_blocks,
-    int q_weight_stride) {
+    int q_weight_stride, int v_unit_norm, float v_eps) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int side = 64 / L;  // heads side by side in a pass
@@ -159,14 +160,22 @@ __global__ __launch_bounds__(kThreads) void attention_prep_kernel(
             if (!store || values_elsewhere) return;
             const int g = unit - n_heads_all;
             const float lam = (v_other && mix) ? mix[0] : 0.f;
-            for (int j = lane; j < D; j += 64) {
-                float v = 0.f;
-                if (j < vdim) {
-                    v = to_float(row[v_off + g * vdim + j]);
-                    if (v_other) v = fmaf(lam, to_float(v_other[static_cast<int64_t>(t) * v_other_stride + g * vdim + j]), (1.0f - lam) * v);
+            auto value = [&](int j) {
+                float v = to_float(row[v_off + g * vdim + j]);
+                if (v_other) v = fmaf(lam, to_float(v_other[static_cast<int64_t>(t) * v_other_stride + g * vdim + j]), (1.0f - lam) * v);
+                return v;
+            };
+            float unit = 1.f;
+            if (v_unit_norm) {  // the head's values divided by their root mean square, as they are cached
+                float sum = 0.f;
+                for (int j = lane; j < vdim; j += 64) {
+                    const float v = value(j);
+                    sum = fmaf(v, v, sum);
                 }
-                v_pool[((page * kv_heads + g) * D + j) * page_size + off] = from_float<T>(v);
+                unit = 1.0f / sqrtf(wave_sum(sum) / static_cast<float>(vdim) + v_eps);
             }
+            for (int j = lane; j < D; j += 64)
+                v_pool[((page * kv_heads + g) * D + j) * page_size + off] = from_float<T>(j < vdim ? value(j) * unit : 0.f);
         } else if (unit == heads + 2 * kv_heads && gate) {
             for (int h = lane; h < heads; h += 64)
                 gate[static_cast<int64_t>(t) * heads + h] = 1.0f / (1.0f + expf(-to_float(row[g_off + h])));
@@ -247,7 +256,7 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
                                    float eps, int pairs, const float* cos_sin, const void* v_other, int64_t v_other_stride,
                                    const float* mix, void* q_out, float* gate, const int32_t* slots, void* k_pool,
                                    void* v_pool, int page_size, int64_t pool_slots, int n_tokens, int dtype,
-                                   int q_weight_stride, hipStream_t stream) {
+                                   int q_weight_stride, int v_unit_norm, float v_eps, hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0 && D >= dim && D >= vdim,
                  "attention_prep: bad sizes heads=%d kv=%d dim=%d vdim=%d D=%d", heads, kv_heads, dim, vdim, D);
     FSIE_REQUIRE(pairs >= 0 && 2 * pairs <= dim && (pairs == 0 || cos_sin), "attention_prep: %d rotated pairs in heads of %d",
@@ -263,7 +272,8 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
     const bool vec = D <= 256 && mult4(q_weight_stride) && mult4(stride) && mult4(q_off) && mult4(k_off) && mult4(dim) && mult4(D) && mult4(pairs) && al16(proj) &&
                      al16(q_out) && al16(k_pool) && al16(q_weight) && al16(k_weight) && al16(cos_sin);
     // portions of prompts in bfloat16: the values go through the kernel that writes eight slots at once
-    const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= kPortionTokens && al16(v_pool)) ? 1 : 0;
+    // (not where the values are normed: that takes a head's values together)
+    const int values_elsewhere = (k_pool && dtype == FSIE_BF16 && n_tokens >= kPortionTokens && al16(v_pool) && !v_unit_norm) ? 1 : 0;
     // many tokens: four units a wave (see the kernel); few: one, so that a decode step has waves enough
     const int hpw = n_tokens >= kPortionTokens ? 4 : 1;
     const int lanes = vec ? (D <= 64 ? 16 : (D <= 128 ? 32 : 64)) : 64;  // lanes a head
@@ -279,7 +289,7 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
         static_cast<const T*>(proj), stride, q_off, k_off, v_off, g_off, heads, kv_heads, dim, vdim, D, q_weight, k_weight, \
         eps, pairs, reinterpret_cast<const float2*>(cos_sin), static_cast<const T*>(v_other), v_other_stride, mix,       \
         static_cast<T*>(q_out), gate, slots, static_cast<T*>(k_pool), static_cast<T*>(v_pool), page_size, pool_slots,   \
-        values_elsewhere, lanes, head_blocks, q_weight_stride)
+        values_elsewhere, lanes, head_blocks, q_weight_stride, v_unit_norm, v_eps)
 #define FSIE_PREP_V(T, V) \
     if (hpw == 4) FSIE_PREP_H(T, V, 4); else FSIE_PREP_H(T, V, 1)
 #define FSIE_PREP(T) \

@@ -53,7 +53,9 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_pages, const int32_t* __restrict__ items,
     T* __restrict__ out, float* __restrict__ partials, int n_heads, int n_kv, int hd, int page_size,
-    int window, float scale, int gh, int head_chunks, const float* __restrict__ sinks, float softcap) {
+    int window, float scale, int gh, int head_chunks, const float* __restrict__ sinks, float softcap,
+    const T* __restrict__ k_pooled, const T* __restrict__ v_pooled, const int32_t* __restrict__ pooled_tables,
+    int pooled_max_pages, int pooled_page_size, int pooled_tokens) {
     extern __shared__ float lds[];
     float* qs = lds;                          // [kRows][hd]
     float* kv = qs + kRows * hd;              // [kKeys][hd + 1]
@@ -71,8 +73,13 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
     if (n_q <= 0) return;  // padding item
     // the first keys that a window keeps: seen whatever the window says, and read before the item's own
     // range where the item is told to
-    const int keep = item[FSIE_ATTN_ITEM_KEEP] & ~FSIE_ATTN_KEEP_WALK;
+    const int keep = item[FSIE_ATTN_ITEM_KEEP] & ~(FSIE_ATTN_KEEP_WALK | FSIE_ATTN_POOL_WALK);
     const int prefix_end = (item[FSIE_ATTN_ITEM_KEEP] & FSIE_ATTN_KEEP_WALK) ? min(keep, key_begin) : 0;
+    // pooled blocks: beside its own keys the item reads one mean key and value for every block of `pooled_tokens`
+    // positions that lies wholly before the window of a query: block b is seen by the query at position p if
+    // (b + 1) * pooled_tokens <= p - window + 1.  They live in pools of their own, an entry a block.
+    const bool pool_walk = k_pooled && (item[FSIE_ATTN_ITEM_KEEP] & FSIE_ATTN_POOL_WALK);
+    const int pooled_end = pool_walk ? max(0, pos0 + n_q - window) / pooled_tokens : 0;
 
     const int group = n_heads / n_kv;
     const int kvh = blockIdx.y / head_chunks;
@@ -107,11 +114,20 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
         for (int i = 0; i < MAXC; ++i) acc[p][i] = 0.f;
     }
     const int n_chunks = (hd + 31) / 32;
-    const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
+    const int32_t* own_table = block_tables + static_cast<int64_t>(seq) * max_pages;
+    const int own_page_size = page_size;
+    const T* const own_k = k_pool;
+    const T* const own_v = v_pool;
 
-    for (int seg = prefix_end > 0 ? 0 : 1; seg < 2; ++seg) {
-    const int seg_begin = seg ? key_begin : 0, seg_end = seg ? key_end : prefix_end;
-    const bool slots_by_four = VEC && (seg_begin & 3) == 0;
+    // three runs of keys: the kept first ones, the item's own range, the pooled blocks
+    for (int seg = prefix_end > 0 ? 0 : 1; seg < (pooled_end > 0 ? 3 : 2); ++seg) {
+    const bool pooled = seg == 2;
+    const int seg_begin = seg == 1 ? key_begin : 0, seg_end = seg == 1 ? key_end : (pooled ? pooled_end : prefix_end);
+    const int32_t* table = pooled ? pooled_tables + static_cast<int64_t>(seq) * pooled_max_pages : own_table;
+    const int page_size = pooled ? pooled_page_size : own_page_size;
+    const T* const k_pool = pooled ? k_pooled : own_k;
+    const T* const v_pool = pooled ? v_pooled : own_v;
+    const bool slots_by_four = VEC && (seg_begin & 3) == 0 && (page_size & 3) == 0;
     for (int kt = seg_begin; kt < seg_end; kt += kKeys) {
         __syncthreads();  // previous tile's values are no longer read (first pass: qs is written)
         if (VEC) {
@@ -151,6 +167,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
             const int pos = pos0 + r / gh;
             const int kj = kt + lane32;
             bool visible = row_ok && kj < seg_end && kj <= pos && (window <= 0 || kj > pos - window || kj < keep);
+            if (pooled) visible = row_ok && kj < seg_end && (kj + 1) * pooled_tokens <= pos - window + 1;
             if (visible) visible = table[kj / page_size] >= 0;
             float s = -INFINITY;
             if (visible) {
@@ -379,6 +396,37 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     }
 }
 
+// One workgroup a job and kv head, a thread a dimension (in turns): the sums run over the block's positions in order.
+template <typename T>
+__global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ k_pool, const T* __restrict__ v_pool,
+                                                          const int32_t* __restrict__ block_tables, int max_pages,
+                                                          int page_size, T* __restrict__ k_pooled, T* __restrict__ v_pooled,
+                                                          const int32_t* __restrict__ pooled_tables, int pooled_max_pages,
+                                                          int pooled_page_size, const int32_t* __restrict__ jobs,
+                                                          int block_tokens, int n_kv, int hd) {
+    const int seq = jobs[2 * blockIdx.x], block = jobs[2 * blockIdx.x + 1];
+    if (seq < 0) return;
+    const int kvh = blockIdx.y;
+    const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
+    const int to_page = pooled_tables[static_cast<int64_t>(seq) * pooled_max_pages + block / pooled_page_size];
+    if (to_page < 0) return;
+    const int to_off = block % pooled_page_size;
+    const float inv = 1.0f / static_cast<float>(block_tokens);
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float ks = 0.f, vs = 0.f;
+        for (int i = 0; i < block_tokens; ++i) {
+            const int pos = block * block_tokens + i;
+            const int page = table[pos / page_size];
+            if (page < 0) continue;
+            const int off = pos % page_size;
+            ks += to_float(k_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + off) * hd + d]);
+            vs += to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + off]);
+        }
+        k_pooled[((static_cast<int64_t>(to_page) * n_kv + kvh) * pooled_page_size + to_off) * hd + d] = from_float<T>(ks * inv);
+        v_pooled[((static_cast<int64_t>(to_page) * n_kv + kvh) * hd + d) * pooled_page_size + to_off] = from_float<T>(vs * inv);
+    }
+}
+
 template <typename T>
 void launch_merge(const float* partials, const int32_t* merges, int n_merges, T* out, int n_heads, int hd, const float* sinks,
                   hipStream_t stream) {
@@ -395,7 +443,12 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
                                      const int32_t* block_tables, int max_pages, const int32_t* items,
                                      int n_items, void* out, float* partials, int n_heads, int n_kv,
                                      int head_dim, int page_size, int window, float scale, int dtype,
-                                     const float* sinks, float softcap, hipStream_t stream) {
+                                     const float* sinks, float softcap, const void* k_pooled, const void* v_pooled,
+                                     const int32_t* pooled_tables, int pooled_max_pages, int pooled_page_size,
+                                     int pooled_tokens, hipStream_t stream) {
+    FSIE_REQUIRE(!k_pooled || (v_pooled && pooled_tables && pooled_max_pages > 0 && pooled_page_size > 0 && pooled_tokens > 0 &&
+                               window > 0),
+                 "attention: pooled blocks come with their pools, tables, a block size and a window");
     FSIE_REQUIRE(n_items >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
                  "attention: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
     FSIE_REQUIRE(head_dim > 0 && head_dim <= 32 * kMaxChunksWide, "attention: head_dim %d must be in 1..%d",
@@ -409,7 +462,8 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
     const dim3 grid(n_items, n_kv * head_chunks);
     const size_t lds = sizeof(float) * (static_cast<size_t>(kRows) * head_dim + kKeys * (head_dim + 1) + kRows * kKeys);
     const bool vec = head_dim % 4 == 0 && page_size % 4 == 0 && reinterpret_cast<uintptr_t>(k_pool) % 16 == 0 &&
-                     reinterpret_cast<uintptr_t>(v_pool) % 16 == 0;
+                     reinterpret_cast<uintptr_t>(v_pool) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pooled) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(v_pooled) % 16 == 0;
     const bool wide = head_dim > 32 * kMaxChunks;
 #define FSIE_SCALAR_ATTENTION(T, VEC, MAXC)                                                                          \
     do {                                                                                                             \
@@ -423,7 +477,9 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
         kernel<<<grid, 256, lds, stream>>>(static_cast<const T*>(q), q_stride, static_cast<const T*>(k_pool),        \
                                            static_cast<const T*>(v_pool), block_tables, max_pages, items,            \
                                            static_cast<T*>(out), partials, n_heads, n_kv, head_dim, page_size, window, \
-                                           scale, gh, head_chunks, sinks, softcap);                                  \
+                                           scale, gh, head_chunks, sinks, softcap, static_cast<const T*>(k_pooled),  \
+                                           static_cast<const T*>(v_pooled), pooled_tables, pooled_max_pages,         \
+                                           pooled_page_size, pooled_tokens);                                         \
     } while (0)
 #define FSIE_SCALAR_ATTENTION_OF(T)                                          \
     if (wide) {                                                              \
@@ -441,6 +497,32 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
 #undef FSIE_SCALAR_ATTENTION_OF
 #undef FSIE_SCALAR_ATTENTION
     FSIE_CHECK_LAUNCH("attention_scalar");
+    return 0;
+}
+
+extern "C" int fsie_pool_blocks(const void* k_pool, const void* v_pool, const int32_t* block_tables, int max_pages,
+                                int page_size, void* k_pooled, void* v_pooled, const int32_t* pooled_tables,
+                                int pooled_max_pages, int pooled_page_size, const int32_t* jobs, int n_jobs, int block_tokens,
+                                int n_kv, int head_dim, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(k_pool && v_pool && block_tables && k_pooled && v_pooled && pooled_tables && jobs, "pool_blocks: missing operand");
+    FSIE_REQUIRE(n_jobs >= 0 && max_pages > 0 && page_size > 0 && pooled_max_pages > 0 && pooled_page_size > 0 &&
+                     block_tokens > 0 && n_kv > 0 && n_kv <= 65535 && head_dim > 0,
+                 "pool_blocks: bad sizes");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "pool_blocks: unknown dtype %d", dtype);
+    if (n_jobs == 0) return 0;
+    const dim3 grid(n_jobs, n_kv);
+    const int threads = head_dim <= 64 ? 64 : (head_dim <= 128 ? 128 : 256);
+    if (dtype == FSIE_F32)
+        pool_blocks_kernel<float><<<grid, threads, 0, stream>>>(
+            static_cast<const float*>(k_pool), static_cast<const float*>(v_pool), block_tables, max_pages, page_size,
+            static_cast<float*>(k_pooled), static_cast<float*>(v_pooled), pooled_tables, pooled_max_pages, pooled_page_size, jobs,
+            block_tokens, n_kv, head_dim);
+    else
+        pool_blocks_kernel<bf16_t><<<grid, threads, 0, stream>>>(
+            static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), block_tables, max_pages, page_size,
+            static_cast<bf16_t*>(k_pooled), static_cast<bf16_t*>(v_pooled), pooled_tables, pooled_max_pages, pooled_page_size,
+            jobs, block_tokens, n_kv, head_dim);
+    FSIE_CHECK_LAUNCH("pool_blocks");
     return 0;
 }
 

@@ -104,7 +104,8 @@ extern "C" int fsie_attention_split_static(const void* q, int64_t q_stride, cons
     int rc = mfma ? fsie_attention_mfma(q, q_stride, k_pool, v_pool, block_tables, max_pages, items_in, n_items, out,
                                         partials, n_heads, n_kv, head_dim, page_size, window, scale, 0, waves, nullptr, 0.f, stream)
                   : fsie_attention_scalar(q, q_stride, k_pool, v_pool, block_tables, max_pages, items_in, n_items, out,
-                                          partials, n_heads, n_kv, head_dim, page_size, window, scale, dtype, nullptr, 0.f, stream);
+                                          partials, n_heads, n_kv, head_dim, page_size, window, scale, dtype, nullptr, 0.f, nullptr,
+                                          nullptr, nullptr, 0, 0, 0, stream);
     if (rc) return rc;
     return fsie_attention_merge(partials, merges_in, n_merges, out, n_heads, head_dim, dtype, nullptr, stream);
 }

@@ -52,9 +52,11 @@ __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
 }
 
 // ---- the activation of a gated feed-forward's gate ---------------------------------------
-// 0: SiLU, g / (1 + exp(-g)); 1: GELU in its tanh form, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).
-enum FsieGateAct { FSIE_ACT_SILU = 0, FSIE_ACT_GELU_TANH = 1 };
+// 0: SiLU, g / (1 + exp(-g)); 1: GELU in its tanh form, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))); 2: max(g, 0).
+enum FsieGateAct { FSIE_ACT_SILU = 0, FSIE_ACT_GELU_TANH = 1, FSIE_ACT_RELU = 2 };
+#define FSIE_ACT_KNOWN(act) ((act) == FSIE_ACT_SILU || (act) == FSIE_ACT_GELU_TANH || (act) == FSIE_ACT_RELU)
 __device__ __forceinline__ float gate_act(float g, int act) {
+    if (act == FSIE_ACT_RELU) return fmaxf(g, 0.f);
     if (act == FSIE_ACT_GELU_TANH) {
         const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
         return 0.5f * g * (1.0f + tanhf(z));

@@ -288,6 +288,19 @@ __global__ void residual_add_kernel(float* __restrict__ residual, const T* __res
 }
 
 template <typename T>
+__global__ void round_to_kernel(const float* __restrict__ x, T* __restrict__ y, int64_t total) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < total) y[i] = from_float<T>(x[i]);
+}
+
+template <typename T>
+__global__ void scaled_sum_kernel(const T* __restrict__ x1, float a, const T* __restrict__ x2, float b, T* __restrict__ y,
+                                  int64_t total) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < total) y[i] = from_float<T>(fmaf(a, to_float(x1[i]), b * to_float(x2[i])));
+}
+
+template <typename T>
 __global__ void bias_add_kernel(T* __restrict__ y, const float* __restrict__ bias, int64_t total, int cols) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < total) y[i] = from_float<T>(to_float(y[i]) + bias[i % cols]);
@@ -516,7 +529,7 @@ extern "C" int fsie_rmsnorm(float* residual, const void* delta, const float* wei
 
 extern "C" int fsie_gated_act(const void* x, void* out, int n_tokens, int inter, int dtype, int act, hipStream_t stream) {
     FSIE_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
-    FSIE_REQUIRE(act == FSIE_ACT_SILU || act == FSIE_ACT_GELU_TANH, "gated_act: unknown activation %d", act);
+    FSIE_REQUIRE(FSIE_ACT_KNOWN(act), "gated_act: unknown activation %d", act);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "swiglu: unknown dtype %d", dtype);
     const int64_t total = static_cast<int64_t>(n_tokens) * inter;
     if (total == 0) return 0;
@@ -536,6 +549,33 @@ extern "C" int fsie_gated_act(const void* x, void* out, int n_tokens, int inter,
 
 extern "C" int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream) {
     return fsie_gated_act(x, out, n_tokens, inter, dtype, FSIE_ACT_SILU, stream);
+}
+
+extern "C" int fsie_round_to(const float* x, void* y, int64_t total, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(total >= 0 && x && y, "round_to: bad operands");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "round_to: unknown dtype %d", dtype);
+    if (total == 0) return 0;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(total, kThreads));
+    if (dtype == FSIE_F32) round_to_kernel<float><<<grid, kThreads, 0, stream>>>(x, static_cast<float*>(y), total);
+    else round_to_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(x, static_cast<bf16_t*>(y), total);
+    FSIE_CHECK_LAUNCH("round_to");
+    return 0;
+}
+
+extern "C" int fsie_scaled_sum(const void* x1, float a, const void* x2, float b, void* y, int64_t total, int dtype,
+                               hipStream_t stream) {
+    FSIE_REQUIRE(total >= 0 && x1 && x2 && y, "scaled_sum: bad operands");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "scaled_sum: unknown dtype %d", dtype);
+    if (total == 0) return 0;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(total, kThreads));
+    if (dtype == FSIE_F32)
+        scaled_sum_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x1), a, static_cast<const float*>(x2), b,
+                                                                static_cast<float*>(y), total);
+    else
+        scaled_sum_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x1), a, static_cast<const bf16_t*>(x2),
+                                                                 b, static_cast<bf16_t*>(y), total);
+    FSIE_CHECK_LAUNCH("scaled_sum");
+    return 0;
 }
 
 extern "C" int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream) {

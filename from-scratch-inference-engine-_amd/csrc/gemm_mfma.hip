@@ -4,7 +4,7 @@
 
 // bfloat16 only.  M <= 64, K a multiple of 8, x and w 16-byte aligned.
 // waves (K split inside a workgroup) and blocks (16-row blocks of W per workgroup): 0 = choose.
-// epilogue: 0 = y = d (+ bias); 1 = SiLU*up over interleaved gate/up rows (N even, no bias, y is [M, N/2]);
+// epilogue: 0 = y = d (+ bias); 3 = the same as 1 with max(gate, 0) on the gate; 1 = SiLU*up over interleaved gate/up rows (N even, no bias, y is [M, N/2]);
 // 2 = the same with GELU (tanh form) for SiLU.
 // splits > 1: K is cut into that many slices, each summed by workgroups of its own; y is then
 // float32 [splits, M, N], partial sums without bias, which the consumer adds in the order of the slices
@@ -18,7 +18,7 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
                  "gemm_mfma_skinny: partial sums are float32, without bias or epilogue");
     FSIE_REQUIRE(splits == 1 || ((K + splits - 1) / splits + 63) / 64 * 64 * (splits - 1) < K,
                  "gemm_mfma_skinny: K=%d is too short for %d slices", K, splits);
-    FSIE_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_mfma_skinny: unknown epilogue %d", epilogue);
+    FSIE_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_mfma_skinny: unknown epilogue %d", epilogue);
     FSIE_REQUIRE(epilogue == 0 || (N % 2 == 0 && !bias && !out_f32),
                  "gemm_mfma_skinny: the SiLU*up epilogue needs an even N, no bias and a bfloat16 result");
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -60,7 +60,7 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
     }
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
     fsie_mm::Call call{x, w, bias, y, M, N, K, splits, stream, fsie_mm::RopeArgs{}};
-    call.act = epilogue == 2 ? FSIE_ACT_GELU_TANH : FSIE_ACT_SILU;
+    call.act = epilogue == 3 ? FSIE_ACT_RELU : (epilogue == 2 ? FSIE_ACT_GELU_TANH : FSIE_ACT_SILU);
     if (epilogue != 0) return fsie_mm::launch_swiglu(blocks, waves, call);
     return out_f32 ? fsie_mm::launch_f32(mt, blocks, waves, call) : fsie_mm::launch_bf16(blocks, waves, call);
 }

@@ -452,7 +452,7 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
 // act: the gate's activation (FsieGateAct: 0 SiLU, 1 GELU in its tanh form).
 extern "C" int fsie_gemm_mfma_wide_gated(const void* x, const void* w, void* y, int M, int N, int K, int waves,
                                          int blocks, int frags, int act, hipStream_t stream) {
-    FSIE_REQUIRE(act == FSIE_ACT_SILU || act == FSIE_ACT_GELU_TANH, "gemm_mfma_wide_gated: unknown activation %d", act);
+    FSIE_REQUIRE(FSIE_ACT_KNOWN(act), "gemm_mfma_wide_gated: unknown activation %d", act);
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide_swiglu: bad sizes M=%d N=%d K=%d", M, N, K);
     FSIE_REQUIRE(M <= (frags ? FSIE_GEMM_MFMA_WIDE_MAX_M : FSIE_GEMM_MFMA_SKINNY_MAX_M),
                  "gemm_mfma_wide_swiglu: at most %d rows (%d on a fragment-ordered weight), got %d",

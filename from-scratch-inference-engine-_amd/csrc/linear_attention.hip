@@ -50,7 +50,8 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 template <typename T>
 __global__ void gla_prep_kernel(const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off,
                                 const float* __restrict__ z, float* __restrict__ prep, int64_t total, int heads, int dim,
-                                int dp, float q_scale, float inv_tau, const int32_t* __restrict__ q_starts, int short_only) {
+                                int dp, float q_scale, float inv_tau, const int32_t* __restrict__ q_starts, int short_only,
+                                const float* __restrict__ head_decay) {
     int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (short_only > 0) {
         const int lo = q_starts[blockIdx.y], len = q_starts[blockIdx.y + 1] - lo;
@@ -67,7 +68,7 @@ __global__ void gla_prep_kernel(const T* __restrict__ proj, int64_t proj_stride,
         const T* row = proj + t * proj_stride + h * dim + i;
         q = to_float(row[q_off]) * q_scale;
         k = to_float(row[k_off]);
-        a = expf(inv_tau * log_sigmoid(z[(t * heads + h) * dim + i]));
+        a = head_decay ? head_decay[h] : expf(inv_tau * log_sigmoid(z[(t * heads + h) * dim + i]));
     }
     prep[e] = q;
     prep[total + e] = k;
@@ -157,7 +158,7 @@ template <typename T>
 __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off, const float* __restrict__ z,
     float* __restrict__ work, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots, int n_seqs,
-    int heads, int dim, int dp, float q_scale, float inv_tau, int n_slots) {
+    int heads, int dim, int dp, float q_scale, float inv_tau, int n_slots, const float* __restrict__ head_decay) {
     extern __shared__ float lds[];  // [3][16][dp + 4]: q, k, B
     const int ld = dp + 4;
     float* qs = lds;
@@ -187,7 +188,8 @@ __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
             const T* row = proj + static_cast<int64_t>(t0 + t) * proj_stride + h * dim + c;
             q = to_float(row[q_off]) * q_scale;
             k = to_float(row[k_off]);
-            la = to_log2 * log_sigmoid(z[(static_cast<int64_t>(t0 + t) * heads + h) * dim + c]);
+            la = head_decay ? log2f(head_decay[h])
+                            : to_log2 * log_sigmoid(z[(static_cast<int64_t>(t0 + t) * heads + h) * dim + c]);
         }
         qs[t * ld + c] = q;
         ks[t * ld + c] = k;
@@ -201,7 +203,14 @@ __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
             sum += bs[t * ld + c];
             bs[t * ld + c] = sum;
         }
-        g[c] = __builtin_amdgcn_exp2f(sum);
+        float whole = __builtin_amdgcn_exp2f(sum);
+        if (head_decay && c < dim) {
+            // a fixed decay: the chunk's decay is its power, by multiplications (it is what the state carries from
+            // chunk to chunk, so its rounding adds up over a long prompt)
+            whole = 1.f;
+            for (int t = 0; t < nt; ++t) whole *= head_decay[h];
+        }
+        g[c] = whole;
     }
     __syncthreads();
     for (int e = tid; e < kGlaChunk * dp; e += kGlaChunkThreads) {
@@ -288,11 +297,12 @@ extern "C" int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_float
 extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* z,
                              float* state, const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens,
                              float* prep, float* out, float* chunk_work, int max_chunks, int heads, int dim, int vdim,
-                             float q_scale, float inv_tau, int n_slots, int dtype, hipStream_t stream) {
+                             float q_scale, float inv_tau, int n_slots, int dtype, const float* head_decay,
+                             hipStream_t stream) {
     FSIE_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && heads > 0 && dim > 0 && vdim > 0 && n_slots > 0, "gla_scan: bad sizes");
     FSIE_REQUIRE(dim <= 256, "gla_scan: %d key channels a head are more than the kernel takes (256)", dim);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gla_scan: unknown dtype %d", dtype);
-    FSIE_REQUIRE(proj && z && state && q_starts && seq_slots && out && prep, "gla_scan: missing operand");
+    FSIE_REQUIRE(proj && (z || head_decay) && state && q_starts && seq_slots && out && prep, "gla_scan: missing operand");
     FSIE_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + heads * dim <= proj_stride &&
                      k_off + heads * dim <= proj_stride && v_off + heads * vdim <= proj_stride,
                  "gla_scan: the q, k and v columns do not fit a row of %lld", static_cast<long long>(proj_stride));
@@ -336,7 +346,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
                                                                dp, splits, n_slots, skip_from)
 #define FSIE_GLA_BY_ROWS(T)                                                                                          \
     gla_prep_kernel<T><<<prep_grid, 256, 0, stream>>>(static_cast<const T*>(proj), proj_stride, q_off, k_off, z, prep, \
-                                                      plane, heads, dim, dp, q_scale, inv_tau, q_starts, short_only); \
+                                                      plane, heads, dim, dp, q_scale, inv_tau, q_starts, short_only, head_decay); \
     if (rows == 1) FSIE_GLA_LAUNCH(T, 1);                                                                            \
     else if (rows == 2) FSIE_GLA_LAUNCH(T, 2);                                                                       \
     else if (rows == 4) FSIE_GLA_LAUNCH(T, 4);                                                                       \
@@ -345,7 +355,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     if (chunks) {                                                                                                    \
         gla_chunk_prep_kernel<T><<<chunk_grid, kGlaChunkThreads, chunk_lds, stream>>>(                                \
             static_cast<const T*>(proj), proj_stride, q_off, k_off, z, chunk_work, q_starts, seq_slots, n_seqs, heads, dim, \
-            dp, q_scale, inv_tau, n_slots);                                                                          \
+            dp, q_scale, inv_tau, n_slots, head_decay);                                                              \
         if (scan_waves == 1) FSIE_GLA_CHUNKS(T, 1);                                                                  \
         else if (scan_waves == 2) FSIE_GLA_CHUNKS(T, 2);                                                             \
         else if (scan_waves == 4) FSIE_GLA_CHUNKS(T, 4);                                                             \

@@ -23,11 +23,14 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int kMaxExperts = 256;
 constexpr int kMaxTop = 16;
 
+// kind 0: scores are sigmoids of the logits; 1: their softmax over all experts.  groups > 1: the experts form that many
+// equal groups of neighbours, a group's score is its largest score (+ correction), and only experts of the `keep` best
+// groups can be chosen.  renorm: the chosen scores are divided by their sum.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router,
                                                         const float* __restrict__ correction, int32_t* __restrict__ ids,
                                                         float* __restrict__ weights, int n_tokens, int hidden, int experts,
-                                                        int top, float scale) {
+                                                        int top, float scale, int kind, int groups, int keep, int renorm) {
     __shared__ float s_score[4][kMaxExperts], s_choice[4][kMaxExperts];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + wave;
@@ -45,14 +48,52 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
         for (int i = 0; i < kWaveDots; ++i)
             if (lane == i) mine = z[i];
         if (lane < kWaveDots && e0 + lane < experts) {
-            const float sc = 1.0f / (1.0f + expf(-mine));
+            const float sc = kind == 1 ? mine : 1.0f / (1.0f + expf(-mine));  // (softmax: the logit for now)
             score[e0 + lane] = sc;
-            choice[e0 + lane] = sc + correction[e0 + lane];
+            choice[e0 + lane] = sc + (correction ? correction[e0 + lane] : 0.f);
+        }
+    }
+    __syncthreads();
+    if (kind == 1 && live) {
+        // every lane reads all logits (the same walk in every lane), then each writes the experts it owns
+        float m = -INFINITY, sum = 0.f;
+        for (int e = 0; e < experts; ++e) m = fmaxf(m, score[e]);
+        for (int e = 0; e < experts; ++e) sum += expf(score[e] - m);
+        float mine[kMaxExperts / 64];
+#pragma unroll
+        for (int i = 0; i < kMaxExperts / 64; ++i) mine[i] = lane + 64 * i < experts ? expf(score[lane + 64 * i] - m) / sum : 0.f;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < kMaxExperts / 64; ++i) {
+            const int e = lane + 64 * i;
+            if (e < experts) {
+                score[e] = mine[i];
+                choice[e] = mine[i] + (correction ? correction[e] : 0.f);
+            }
         }
     }
     __syncthreads();
     if (!live) return;
     // every lane walks the same choice (a few experts, a few picks): no exchange needed
+    unsigned long long kept[kMaxExperts / 64];
+#pragma unroll
+    for (int i = 0; i < kMaxExperts / 64; ++i) kept[i] = ~0ull;
+    const int per_group = groups > 1 ? experts / groups : experts;
+    if (groups > 1 && keep < groups) {
+#pragma unroll
+        for (int i = 0; i < kMaxExperts / 64; ++i) kept[i] = 0ull;
+        for (int c = 0; c < keep; ++c) {
+            int best = -1;
+            float best_v = -INFINITY;
+            for (int g = 0; g < groups; ++g) {
+                if ((kept[g >> 6] >> (g & 63)) & 1ull) continue;
+                float v = -INFINITY;
+                for (int e = g * per_group; e < (g + 1) * per_group; ++e) v = fmaxf(v, choice[e]);
+                if (best < 0 || v > best_v) best = g, best_v = v;
+            }
+            kept[best >> 6] |= 1ull << (best & 63);
+        }
+    }
     int picked[kMaxTop];
     float chosen[kMaxTop];
     float total = 0.f;
@@ -62,7 +103,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
         for (int e = 0; e < experts; ++e) {
             bool taken = false;
             for (int p = 0; p < c; ++p) taken = taken || picked[p] == e;
-            const float v = choice[e];
+            const int g = e / per_group;
+            const bool allowed = groups <= 1 || ((kept[g >> 6] >> (g & 63)) & 1ull);
+            const float v = allowed ? choice[e] : -INFINITY;
             if (!taken && (best < 0 || v > best_v)) best = e, best_v = v;
         }
         picked[c] = best;
@@ -75,7 +118,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
         for (int c = 0; c < top; ++c)
             if (c == lane) mine = chosen[c], id = picked[c];
         ids[static_cast<int64_t>(t) * top + lane] = id;
-        weights[static_cast<int64_t>(t) * top + lane] = mine / (total + 1e-20f) * scale;
+        weights[static_cast<int64_t>(t) * top + lane] = renorm ? mine / (total + 1e-20f) * scale : mine * scale;
     }
 }
 
@@ -345,8 +388,15 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
                 const int n = n0 + 16 * j + r;
                 if (n >= N) continue;
                 const float v = acc[i][j][u];
-                if (epilogue == 1) static_cast<float*>(out)[slot * N + n] = v * scale;
-                else static_cast<T*>(out)[slot * N + n] = from_float<T>(gelu_erf(v));
+                if (epilogue == 1) {
+                    static_cast<float*>(out)[slot * N + n] = v * scale;
+                } else if (epilogue >= 2) {
+                    // gate and up rows in turn: the even output's neighbour lane holds its up value
+                    const float up = __shfl_xor(v, 1, FSIE_WAVE);
+                    if (!(n & 1)) static_cast<T*>(out)[slot * (N / 2) + n / 2] = from_float<T>(gate_act(v, epilogue - 2) * up);
+                } else {
+                    static_cast<T*>(out)[slot * N + n] = from_float<T>(gelu_erf(v));
+                }
             }
         }
     }
@@ -386,21 +436,27 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 }  // namespace
 
 extern "C" int fsie_moe_route(const void* x, const void* router, const float* correction, int dtype, int32_t* ids,
-                              float* weights, int n_tokens, int hidden, int experts, int top, float scale,
-                              hipStream_t stream) {
+                              float* weights, int n_tokens, int hidden, int experts, int top, float scale, int kind,
+                              int groups, int keep, int renorm, hipStream_t stream) {
+    FSIE_REQUIRE(kind == 0 || kind == 1, "moe_route: unknown kind of scores %d", kind);
+    FSIE_REQUIRE(groups >= 1 && experts % groups == 0 && keep >= 1 && keep <= groups &&
+                     (groups == 1 || top <= keep * (experts / groups)),
+                 "moe_route: %d experts in %d groups of which %d are kept do not give %d choices", experts, groups, keep, top);
     FSIE_REQUIRE(n_tokens >= 0 && hidden > 0 && experts > 0 && experts <= kMaxExperts && top > 0 && top <= experts &&
                      top <= kMaxTop, "moe_route: bad sizes T=%d hidden=%d experts=%d (at most %d) top=%d (at most %d)",
                  n_tokens, hidden, experts, kMaxExperts, top, kMaxTop);
-    FSIE_REQUIRE(x && router && correction && ids && weights, "moe_route: missing operand");
+    FSIE_REQUIRE(x && router && ids && weights, "moe_route: missing operand");
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "moe_route: unknown dtype %d", dtype);
     if (n_tokens == 0) return 0;
     const unsigned grid = static_cast<unsigned>((n_tokens + 3) / 4);
     if (dtype == FSIE_F32)
         moe_route_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x), static_cast<const float*>(router),
-                                                          correction, ids, weights, n_tokens, hidden, experts, top, scale);
+                                                          correction, ids, weights, n_tokens, hidden, experts, top, scale, kind,
+                                                          groups, keep, renorm);
     else
         moe_route_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(router),
-                                                           correction, ids, weights, n_tokens, hidden, experts, top, scale);
+                                                           correction, ids, weights, n_tokens, hidden, experts, top, scale, kind,
+                                                          groups, keep, renorm);
     FSIE_CHECK_LAUNCH("moe_route");
     return 0;
 }
@@ -433,7 +489,8 @@ extern "C" int fsie_moe_gemm(const void* a, const void* w, void* out, const int3
     FSIE_REQUIRE(tile_rows == 16 || tile_rows == 32 || tile_rows == 64 || tile_rows == 128,
                  "moe_gemm: tiles of %d rows (the kernels take 16, 32, 64, 128)", tile_rows);
     FSIE_REQUIRE(a && w && out && tiles && order, "moe_gemm: missing operand");
-    FSIE_REQUIRE(epilogue == 0 || (epilogue == 1 && pair_weight), "moe_gemm: unknown epilogue %d", epilogue);
+    FSIE_REQUIRE(epilogue == 0 || (epilogue == 1 && pair_weight) || (epilogue >= 2 && FSIE_ACT_KNOWN(epilogue - 2) && N % 2 == 0),
+                 "moe_gemm: unknown epilogue %d", epilogue);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "moe_gemm: unknown dtype %d", dtype);
     if (max_tiles == 0) return 0;
     const int64_t per_die = ceil_div64(max_tiles, 8);

@@ -49,7 +49,8 @@ __global__ __launch_bounds__(kThreads) void sandwich_norm_kernel(
     }
     const float scale = 1.0f / sqrtf(block_sum(sum_sq, scratch) / static_cast<float>(hidden) + eps);
     T* dst = out + static_cast<int64_t>(r) * hidden;
-    for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = from_float<T>((row_buf[j] * scale) * weight[j]);
+    for (int j = threadIdx.x; j < hidden; j += kThreads)
+        dst[j] = from_float<T>(weight ? (row_buf[j] * scale) * weight[j] : row_buf[j]);  // (no weight: the stream itself)
 }
 
 // Four consecutive elements: one 16-byte (float32) or 8-byte (bfloat16) access.
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(THREADS) void sandwich_norm_vec_kernel(
         const int j = min((it * THREADS + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
         v[it] = load4(res + j);
         wp[it] = load4(post_weight + j);
-        w[it] = load4(weight + j);
+        w[it] = weight ? load4(weight + j) : float4{1.f, 1.f, 1.f, 1.f};
         if (del) {
             y[it] = load4(del + j);
         } else {
@@ -120,7 +121,8 @@ __global__ __launch_bounds__(THREADS) void sandwich_norm_vec_kernel(
             sum_sq += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
         }
     }
-    const float scale = 1.0f / sqrtf(block_sum(sum_sq, scratch) / static_cast<float>(hidden) + eps);
+    // without a weight the stream itself is the result (a layer whose sublayers read the stream as it is)
+    const float scale = weight ? 1.0f / sqrtf(block_sum(sum_sq, scratch) / static_cast<float>(hidden) + eps) : 1.f;
     T* dst = out + static_cast<int64_t>(r) * hidden;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
@@ -180,7 +182,7 @@ extern "C" int fsie_sandwich_norm(float* residual, const void* delta, const floa
     FSIE_REQUIRE(n_rows >= 0 && hidden > 0 && hidden <= 16384, "sandwich_norm: bad sizes rows=%d hidden=%d (at most 16384)",
                  n_rows, hidden);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "sandwich_norm: unknown dtype %d", dtype);
-    FSIE_REQUIRE(residual && delta && post_weight && weight && out, "sandwich_norm: missing operand");
+    FSIE_REQUIRE(residual && delta && post_weight && out, "sandwich_norm: missing operand");
     FSIE_REQUIRE(n_parts >= 0 && n_parts <= FSIE_GEMM_MAX_SPLITS, "sandwich_norm: 0 to %d partial sums, got %d",
                  FSIE_GEMM_MAX_SPLITS, n_parts);
     FSIE_REQUIRE(!(write_back && rows), "sandwich_norm: chosen rows are read, not written back");
@@ -233,7 +235,7 @@ extern "C" int fsie_gated_headnorm(const float* o, int n_planes, const void* gat
     FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && width > 0, "gated_headnorm: bad sizes T=%d heads=%d width=%d", n_tokens, heads,
                  width);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gated_headnorm: unknown dtype %d", dtype);
-    FSIE_REQUIRE(act == FSIE_ACT_SILU || act == FSIE_ACT_GELU_TANH, "gated_headnorm: unknown activation %d", act);
+    FSIE_REQUIRE(FSIE_ACT_KNOWN(act), "gated_headnorm: unknown activation %d", act);
     FSIE_REQUIRE(o && gate && weight && out && gate_stride >= static_cast<int64_t>(heads) * width,
                  "gated_headnorm: missing operand or a gate row shorter than the heads");
     if (n_tokens == 0) return 0;

@@ -56,6 +56,18 @@ def block_state_cache(call: int) -> int:
     return -2 - call
 
 
+def _flatten_needs(cid, need, into: Dict, shapes: Dict) -> None:
+    """A mixer that keeps several things for a request returns its needs by name (a dict, which may hold dicts): every
+    need gets the cache id (id, name) and ``shapes`` remembers the names, so that the mixer's ``forward`` gets a dict of
+    views of the same shape."""
+    if isinstance(need, dict):
+        shapes[cid] = list(need)
+        for name, sub in need.items():
+            _flatten_needs((cid, name), sub, into, shapes)
+    elif need is not None:
+        into[cid] = need
+
+
 class Model:
     def __init__(self, spec: ModelSpec, dtype, device):
         self.spec = spec
@@ -65,15 +77,14 @@ class Model:
         self.weight_bytes = 0
         # caches: one per call of the schedule that keeps one
         self.call_cache: List[int] = []
-        needs: Dict[int, object] = {}
+        needs: Dict[object, object] = {}
+        self.cache_shapes: Dict[object, List[str]] = {}
         for i, call in enumerate(spec.schedule):
             if not 0 <= call.layer < len(spec.layers):
                 raise ValueError(f"schedule entry {i} names layer {call.layer}, which does not exist")
             if call.cache_of is None:
                 self.call_cache.append(i)
-                need = spec.layers[call.layer].mixer.cache_need()
-                if need is not None:
-                    needs[i] = need
+                _flatten_needs(i, spec.layers[call.layer].mixer.cache_need(), needs, self.cache_shapes)
                 # what the block itself keeps for a request (the inputs of a convolution in front of its sublayers)
                 own = getattr(spec.layers[call.layer], "state_need", lambda: None)()
                 if own is not None:
@@ -110,15 +121,17 @@ class Model:
             else:
                 states[cid] = need
         self.cache_layout = CacheLayout(groups, group_caches, states)
-        self.cached_calls = set(needs)
-        # planners of all mixers, one per distinct key
+        self.cached_calls = set(needs) | set(self.cache_shapes)
+        # planners of all mixers, one per distinct key (a mixer made of mixers names theirs in ``planners()``)
         self.planners = []
         seen = set()
         for block in spec.layers:
-            planner = block.mixer.planner()
-            if planner is not None and planner.key not in seen:
-                seen.add(planner.key)
-                self.planners.append(planner)
+            mixer = block.mixer
+            mine = mixer.planners() if callable(getattr(mixer, "planners", None)) else [mixer.planner()]
+            for planner in mine:
+                if planner is not None and planner.key not in seen:
+                    seen.add(planner.key)
+                    self.planners.append(planner)
 
     # ---------------------------------------------------------------- construction
     @classmethod
@@ -196,6 +209,12 @@ class Model:
         return max(1, min(pages, (2 ** 31 - 1) // max(1, per_layer * page_size)))
 
     # ---------------------------------------------------------------- compute
+    def _cache_view(self, storage: CacheStorage, cid, ctx: StepContext, writes: bool):
+        names = self.cache_shapes.get(cid)
+        if names is not None:
+            return {name: self._cache_view(storage, (cid, name), ctx, writes) for name in names}
+        return storage.view(cid, ctx, writes=writes)
+
     def forward(self, ctx: StepContext, storage: CacheStorage) -> torch.Tensor:
         """float32 logits [wanted, vocab] for the step described by ``ctx``."""
         spec = self.spec
@@ -207,7 +226,7 @@ class Model:
         hidden = HiddenState(spec.embedding.embed(ctx, kept))
         for i, call in enumerate(spec.schedule):
             cid = self.call_cache[i]
-            cache = storage.view(cid, ctx, writes=call.cache_of is None) if cid in self.cached_calls else None
+            cache = self._cache_view(storage, cid, ctx, call.cache_of is None) if cid in self.cached_calls else None
             own = block_state_cache(i)
             if own in self.cached_calls:
                 spec.layers[call.layer].forward(hidden, ctx, cache, state=storage.view(own, ctx, writes=True))

@@ -31,7 +31,7 @@ def known_architectures():
 
 
 def _ensure_builtin() -> None:
-    from . import botulorn, fiterax, gilozen, qwen2  # noqa: F401  (they register themselves)
+    from . import botulorn, fiterax, gilozen, mafosun, qwen2  # noqa: F401  (they register themselves)
 
 
 def architecture_of(raw: Mapping) -> Architecture:

@@ -14,7 +14,7 @@ from .functions import (FragmentOrdered, attention_merge, attention_mfma, attent
                         rmsnorm, rmsnorm_plain, rope_kv_write, rope_table, sample, swiglu, zero_pages, zero_rows,
                         gate_act_code, gated_headnorm, gla_scan, head_gemm, latent_prep, rope_pairs, sandwich_norm, softcap,
                         attention_prep, gate_heads, layer_norm, pair_embedding,
-                        group_rmsnorm, causal_conv, mlstm_state_floats, mlstm_scan, mlstm_out, moe_route, moe_group, moe_gemm, moe_combine, moe_tile_rows, sum_round, GEMM_AUTO, GEMM_TILED, GEMM_SKINNY, GEMM_NARROW)
+                        group_rmsnorm, causal_conv, mlstm_state_floats, mlstm_scan, mlstm_out, moe_route, moe_group, moe_gemm, moe_combine, moe_tile_rows, sum_round, pool_blocks, scaled_sum, round_to, GEMM_AUTO, GEMM_TILED, GEMM_SKINNY, GEMM_NARROW)
 from .library import KernelError, KernelLibraryMissing, load
 from .tuning import disable_library_tuning, enable_library_tuning, library_mm, library_tuning_enabled
 
@@ -26,4 +26,4 @@ __all__ = ["FragmentOrdered", "KernelError", "KernelLibraryMissing", "attention_
            "rmsnorm", "rmsnorm_plain", "rope_kv_write", "rope_table", "sample", "swiglu", "zero_pages", "zero_rows",
            "gate_act_code", "gated_headnorm", "gla_scan", "head_gemm", "latent_prep", "rope_pairs", "sandwich_norm", "softcap",
            "attention_prep", "gate_heads", "layer_norm", "pair_embedding",
-           "group_rmsnorm", "causal_conv", "mlstm_state_floats", "mlstm_scan", "mlstm_out", "moe_route", "moe_group", "moe_gemm", "moe_combine", "moe_tile_rows", "sum_round", "GEMM_AUTO", "GEMM_TILED", "GEMM_SKINNY", "GEMM_NARROW"]
+           "group_rmsnorm", "causal_conv", "mlstm_state_floats", "mlstm_scan", "mlstm_out", "moe_route", "moe_group", "moe_gemm", "moe_combine", "moe_tile_rows", "sum_round", "pool_blocks", "scaled_sum", "round_to", "GEMM_AUTO", "GEMM_TILED", "GEMM_SKINNY", "GEMM_NARROW"]

@@ -13,6 +13,7 @@ from .library import KernelError, check, load
 F32, BF16 = 0, 1
 ATTN_ITEM_INTS = 8
 ATTN_MERGE_INTS = 4
+ATTN_POOL_WALK = 1 << 29  # the item also reads the pooled blocks before its queries' windows
 ATTN_KEEP_WALK = 1 << 30  # in an item's last field, beside the number of kept first keys: read them before the item's range
 GEMM_SKINNY_MAX_M = 8
 GEMM_MFMA_SKINNY_MAX_M = 64
@@ -162,7 +163,7 @@ def random_fill(out: torch.Tensor, key: int, init: str, std: float = 0.0) -> tor
     return out
 
 
-GATE_ACTS = {"silu": 0, "gelu_tanh": 1}  # the activations of a gate that the kernels know
+GATE_ACTS = {"silu": 0, "gelu_tanh": 1, "relu": 2}  # the activations of a gate that the kernels know
 
 
 def gate_act_code(act: str) -> int:
@@ -340,7 +341,7 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     out_dtype = out_dtype or x.dtype
     if out_dtype not in (torch.bfloat16, torch.float32):
         raise KernelError(f"gemm: output {out_dtype} is not offered")
-    if epilogue not in ("plain", "swiglu", "geglu_tanh"):
+    if epilogue not in ("plain", "swiglu", "geglu_tanh", "reglu"):
         raise KernelError(f"gemm: unknown epilogue '{epilogue}'")
     gated = epilogue != "plain"  # "geglu_tanh": the same with GELU (tanh form) on the gate
     if gated and n % 2:
@@ -356,7 +357,7 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     _need(out, "gemm out", dtype=out_dtype, shape=shape)
     check(load().fsie_gemm_mfma_skinny(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
                                        int(out_dtype == torch.float32), waves, blocks,
-                                       {"plain": 0, "swiglu": 1, "geglu_tanh": 2}[epilogue],
+                                       {"plain": 0, "swiglu": 1, "geglu_tanh": 2, "reglu": 3}[epilogue],
                                        splits, _stream()))
     return out
 
@@ -532,10 +533,12 @@ def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_poo
                      block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
                      partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
                      window: Optional[int], scale: float, n_query_rows: int,
-                     sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> torch.Tensor:
+                     sinks: Optional[torch.Tensor] = None, softcap: float = 0.0, pooled=None) -> torch.Tensor:
     """Attention of the work items over the paged cache (float32 arithmetic).  ``sinks`` (float32 [n_heads],
     here and in the other attention functions): exp(sinks[h]) is one more term of the denominator of
-    head h's softmax, with no key and no value.
+    head h's softmax, with no key and no value.  ``pooled`` = (k_pool, v_pool, block_tables, block_tokens) of the
+    pools of pooled blocks (one mean key and value for every ``block_tokens`` positions): items flagged
+    ``ATTN_POOL_WALK`` also read the blocks that lie wholly before their queries' windows.
 
     ``q`` is a view into rows of stride ``q_stride`` elements whose first n_heads*head_dim columns
     are the queries; ``out`` is [n_query_rows, n_heads*head_dim]."""
@@ -555,12 +558,62 @@ def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_poo
         raise KernelError("attention: q_stride is smaller than the query width")
     if partials is not None:
         _need(partials, "attention partials", dtype=torch.float32, ndim=1)
+    pooled_args = (None, None, None, 0, 0, 0)
+    if pooled is not None:
+        pk, pv, ptab, block_tokens = pooled
+        _need(pk, "pooled k_pool", dtype=q.dtype, ndim=4)
+        _need(pv, "pooled v_pool", dtype=q.dtype, shape=(pk.shape[0], pk.shape[1], pk.shape[3], pk.shape[2]))
+        _need(ptab, "pooled block_tables", dtype=torch.int32, ndim=2)
+        if pk.shape[1] != n_kv or pk.shape[3] != head_dim or ptab.shape[0] != block_tables.shape[0] or not window:
+            raise KernelError("attention: the pools of pooled blocks do not fit the layer (heads, head size, requests, a window)")
+        pooled_args = (pk.data_ptr(), pv.data_ptr(), ptab.data_ptr(), ptab.shape[1], pk.shape[2], int(block_tokens))
     check(load().fsie_attention_scalar(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                        block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
                                        n_items, out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim,
                                        page_size, int(window or 0), float(scale), dtype_code(q.dtype),
-                                       _sinks_ptr(sinks, n_heads), float(softcap or 0.0), _stream()))
+                                       _sinks_ptr(sinks, n_heads), float(softcap or 0.0), *pooled_args, _stream()))
     return out
+
+
+def pool_blocks(k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor, k_pooled: torch.Tensor,
+                v_pooled: torch.Tensor, pooled_tables: torch.Tensor, jobs: torch.Tensor, n_jobs: int, block_tokens: int) -> None:
+    """The mean key and value of every block of ``block_tokens`` positions that ``jobs`` int32 [n, 2] names (request of
+    the step, block; request -1: nothing), read from the pages of keys and values and written to the pools of pooled
+    blocks at the entry of the block (float32 sums in the order of the positions)."""
+    _need(k_pool, "k_pool", ndim=4)
+    units, n_kv, page_size, hd = k_pool.shape
+    _need(v_pool, "v_pool", dtype=k_pool.dtype, shape=(units, n_kv, hd, page_size))
+    _need(k_pooled, "pooled k_pool", dtype=k_pool.dtype, ndim=4)
+    if k_pooled.shape[1] != n_kv or k_pooled.shape[3] != hd:
+        raise KernelError("pool_blocks: the pools of pooled blocks hold other heads")
+    _need(v_pooled, "pooled v_pool", dtype=k_pool.dtype, shape=(k_pooled.shape[0], n_kv, hd, k_pooled.shape[2]))
+    _need(block_tables, "block_tables", dtype=torch.int32, ndim=2)
+    _need(pooled_tables, "pooled block_tables", dtype=torch.int32, ndim=2)
+    _need(jobs, "pool_blocks jobs", dtype=torch.int32, ndim=2)
+    if jobs.shape[1] != 2 or jobs.shape[0] < n_jobs or pooled_tables.shape[0] != block_tables.shape[0]:
+        raise KernelError("pool_blocks: bad tables")
+    check(load().fsie_pool_blocks(k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
+                                  page_size, k_pooled.data_ptr(), v_pooled.data_ptr(), pooled_tables.data_ptr(),
+                                  pooled_tables.shape[1], k_pooled.shape[2], jobs.data_ptr(), int(n_jobs), int(block_tokens),
+                                  n_kv, hd, dtype_code(k_pool.dtype), _stream()))
+
+
+def round_to(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The float32 tensor ``x`` in ``dtype`` (rounded to nearest even; a copy for float32)."""
+    _need(x, "round_to x", dtype=torch.float32)
+    y = torch.empty(x.shape, dtype=dtype, device=x.device)
+    check(load().fsie_round_to(x.data_ptr(), y.data_ptr(), x.numel(), dtype_code(dtype), _stream()))
+    return y
+
+
+def scaled_sum(x1: torch.Tensor, a: float, x2: torch.Tensor, b: float) -> torch.Tensor:
+    """a * x1 + b * x2 in float32, rounded once to the operands' type."""
+    _need(x1, "scaled_sum x1")
+    _need(x2, "scaled_sum x2", dtype=x1.dtype, shape=tuple(x1.shape))
+    y = torch.empty_like(x1)
+    check(load().fsie_scaled_sum(x1.data_ptr(), float(a), x2.data_ptr(), float(b), y.data_ptr(), x1.numel(),
+                                 dtype_code(x1.dtype), _stream()))
+    return y
 
 
 def attention_mfma_rows(head_dim: int, large: bool) -> int:
@@ -738,14 +791,15 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
 # a layer with a norm before and after every sublayer; norms of heads with a gate; the logits' cap
 # ---------------------------------------------------------------------------------------------
 def sandwich_norm(residual: torch.Tensor, delta: torch.Tensor, post_weight: torch.Tensor, post_eps: float,
-                  weight: torch.Tensor, eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                  weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                   write_back: bool = False) -> torch.Tensor:
     """``v = residual + rmsnorm(delta; post_weight, post_eps)``, then ``rmsnorm(v; weight, eps)`` in
     ``out_dtype``, one pass.  ``delta`` as for ``rmsnorm``; ``write_back`` stores v into ``residual``
     (not with ``rows``, which selects the rows to work on)."""
     _need(residual, "sandwich_norm residual", dtype=torch.float32, ndim=2)
     t, h = residual.shape
-    _need(weight, "sandwich_norm weight", dtype=torch.float32, shape=(h,))
+    if weight is not None:  # (None: the result is v itself, rounded to ``out_dtype``)
+        _need(weight, "sandwich_norm weight", dtype=torch.float32, shape=(h,))
     _need(post_weight, "sandwich_norm post weight", dtype=torch.float32, shape=(h,))
     n_parts = 0
     if delta.ndim == 3:
@@ -763,7 +817,7 @@ def sandwich_norm(residual: torch.Tensor, delta: torch.Tensor, post_weight: torc
             raise KernelError("sandwich_norm: chosen rows are not written back")
     out = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device)
     check(load().fsie_sandwich_norm(residual.data_ptr(), delta.data_ptr(), post_weight.data_ptr(), float(post_eps),
-                                    weight.data_ptr(), float(eps), out.data_ptr(), _ptr(rows), n_rows, h,
+                                    _ptr(weight), float(eps), out.data_ptr(), _ptr(rows), n_rows, h,
                                     dtype_code(out_dtype), int(write_back), n_parts, t, _stream()))
     return out
 
@@ -802,7 +856,7 @@ def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
 # ---------------------------------------------------------------------------------------------
 def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, state: torch.Tensor,
              q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int, q_scale: float,
-             inv_tau: float, chunked: bool = True) -> torch.Tensor:
+             inv_tau: float, chunked: bool = True, head_decay: Optional[torch.Tensor] = None) -> torch.Tensor:
     """S <- diag(sigmoid(z_t)^inv_tau) S + k_t v_t^T, o_t = S^T (q_scale q_t) over the tokens of every
     request of the step, from and to ``state`` float32 [slots, heads, dim, vdim].  ``proj`` [T, W] holds the
     q, k (heads x dim) and v (heads x vdim) columns from ``q_off``, ``k_off``, ``v_off``; ``z`` float32
@@ -813,7 +867,11 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
     every portion token by token."""
     _need(proj, "gla proj", ndim=2)
     t, w = proj.shape
-    _need(z, "gla z", dtype=torch.float32, shape=(t, heads * dim))
+    if head_decay is not None:
+        # a fixed decay a head (float32 [heads]) instead of the decays of every token and key channel
+        _need(head_decay, "gla head decay", dtype=torch.float32, shape=(heads,))
+    else:
+        _need(z, "gla z", dtype=torch.float32, shape=(t, heads * dim))
     _need(state, "gla state", dtype=torch.float32, ndim=4)
     if tuple(state.shape[1:]) != (heads, dim, vdim):
         raise KernelError(f"gla state: shape {tuple(state.shape)} is not [slots, {heads}, {dim}, {vdim}]")
@@ -831,10 +889,10 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
     # a step of single tokens (t == n, as every captured decode step is) has no portion to cut into chunks
     max_chunks = t // chunk_tokens.value + n if chunked and t > n and t >= chunk_min.value else 0
     work = torch.empty((max_chunks * chunk_floats.value,), dtype=torch.float32, device=proj.device) if max_chunks else None
-    check(load().fsie_gla_scan(proj.data_ptr(), w, q_off, k_off, v_off, z.data_ptr(), state.data_ptr(), q_starts.data_ptr(),
+    check(load().fsie_gla_scan(proj.data_ptr(), w, q_off, k_off, v_off, _ptr(z), state.data_ptr(), q_starts.data_ptr(),
                                seq_slots.data_ptr(), n, t, prep.data_ptr(), out.data_ptr(),
                                work.data_ptr() if work is not None else None, max_chunks, heads, dim, vdim, float(q_scale),
-                               float(inv_tau), state.shape[0], dtype_code(proj.dtype), _stream()))
+                               float(inv_tau), state.shape[0], dtype_code(proj.dtype), _ptr(head_decay), _stream()))
     return out
 
 
@@ -986,8 +1044,10 @@ def attention_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off
                    vdim: int, padded: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                    pairs: int, cos_sin: Optional[torch.Tensor], gated: bool, v_other: Optional[torch.Tensor] = None,
                    v_other_stride: int = 0, mix: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
-                   k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None):
-    """From the fused projection ``proj`` [T, W] (q, k, v and one gate logit a head at their column offsets): the
+                   k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,
+                   v_unit_norm_eps: Optional[float] = None):
+    """``v_unit_norm_eps`` (a number or None): every kv head's values are divided by sqrt(mean(v^2) + eps) before they
+    are cached.  From the fused projection ``proj`` [T, W] (q, k, v and one gate logit a head at their column offsets): the
     queries [T, heads * padded] after the heads' RMS norm (weights float32 [dim] or None) and the rotation of their
     first ``pairs`` pairs (i, i + pairs) by ``cos_sin`` [T, pairs, 2] (``q_weight`` may also be [heads, dim]: a weight
     of its own for every query head); the gates' sigmoid (float32 [T, heads], or
@@ -1028,7 +1088,7 @@ def attention_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off
                                      _ptr(q_weight), _ptr(k_weight), float(eps), pairs, _ptr(cos_sin), _ptr(v_other),
                                      int(v_other_stride), _ptr(mix), q.data_ptr(), _ptr(gate), _ptr(slots), _ptr(k_pool),
                                      _ptr(v_pool), page_size, pool_slots, t, dtype_code(proj.dtype), q_weight_stride,
-                                     _stream()))
+                                     int(v_unit_norm_eps is not None), float(v_unit_norm_eps or 0.0), _stream()))
     return q, gate
 
 
@@ -1184,21 +1244,29 @@ def moe_tile_rows(n_pairs: int, experts: int) -> int:
     return int(load().fsie_moe_tile_rows(int(n_pairs), int(experts)))
 
 
-def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int, scale: float):
+def moe_route(x: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], top: int, scale: float,
+              scores: str = "sigmoid", groups: int = 1, keep: int = 1, renorm: bool = True):
     """(ids int32 [T, top], weights float32 [T, top]): the ``top`` experts with the largest sigmoid(x . router^T) +
     correction (ties: the lower index) and their weights, the chosen sigmoids divided by their sum times ``scale``.
-    ``x`` [T, H] and ``router`` [E, H] share a type; the logits are summed in float32."""
+    ``x`` [T, H] and ``router`` [E, H] share a type; the logits are summed in float32.  ``scores="softmax"``: the scores
+    are the softmax of the logits over all experts.  ``groups`` > 1: the experts form that many equal groups of
+    neighbours and only those of the ``keep`` groups with the largest best score can be chosen.  ``renorm=False``: the
+    weights are the chosen scores themselves times ``scale``.  ``correction`` may be None."""
     _need(x, "moe_route x", ndim=2)
     t, h = x.shape
     _need(router, "moe_route router", dtype=x.dtype, ndim=2)
     e = router.shape[0]
     if router.shape[1] != h:
         raise KernelError(f"moe_route: router {tuple(router.shape)} does not fit rows of {h}")
-    _need(correction, "moe_route correction", dtype=torch.float32, shape=(e,))
+    if correction is not None:
+        _need(correction, "moe_route correction", dtype=torch.float32, shape=(e,))
+    if scores not in ("sigmoid", "softmax"):
+        raise KernelError(f"moe_route: unknown scores '{scores}'")
     ids = torch.empty((t, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((t, top), dtype=torch.float32, device=x.device)
-    check(load().fsie_moe_route(x.data_ptr(), router.data_ptr(), correction.data_ptr(), dtype_code(x.dtype), ids.data_ptr(),
-                                weights.data_ptr(), t, h, e, int(top), float(scale), _stream()))
+    check(load().fsie_moe_route(x.data_ptr(), router.data_ptr(), _ptr(correction), dtype_code(x.dtype), ids.data_ptr(),
+                                weights.data_ptr(), t, h, e, int(top), float(scale), int(scores == "softmax"), int(groups),
+                                int(keep), int(bool(renorm)), _stream()))
     return ids, weights
 
 
@@ -1219,12 +1287,14 @@ def moe_group(ids: torch.Tensor, experts: int, tile_rows: Optional[int] = None):
 
 
 def moe_gemm(a: torch.Tensor, weight: torch.Tensor, tiles: torch.Tensor, order: torch.Tensor, gather_div: int = 0,
-             pair_weight: Optional[torch.Tensor] = None, tile_rows: Optional[int] = None) -> torch.Tensor:
+             pair_weight: Optional[torch.Tensor] = None, tile_rows: Optional[int] = None,
+             gated: Optional[str] = None) -> torch.Tensor:
     """One product per expert: out[slot] = a[row(slot)] . weight[expert of slot]^T with ``weight`` [E, N, K].
     ``gather_div`` > 0: row(slot) = order[slot] // gather_div (``a`` holds tokens); 0: row(slot) = slot.  Without
     ``pair_weight`` the result is the exact GELU of the product in ``a``'s type; with it (float32 [pairs]) the product
     times the pair's weight, float32.  ``tile_rows``: the rows of a tile of ``tiles`` (default: what ``moe_tile_rows``
-    names for the step, as ``moe_group``'s default is)."""
+    names for the step, as ``moe_group``'s default is).  ``gated`` (a gate activation's name): the rows of every
+    expert's matrix are gate and up in turn and the result is act(gate) * up, [slots, N / 2]."""
     _need(a, "moe_gemm a", ndim=2)
     _need(weight, "moe_gemm weight", dtype=a.dtype, ndim=3)
     _, n, k = weight.shape
@@ -1240,9 +1310,13 @@ def moe_gemm(a: torch.Tensor, weight: torch.Tensor, tiles: torch.Tensor, order: 
         _need(pair_weight, "moe_gemm pair weights", dtype=torch.float32)
         if pair_weight.numel() != slots:
             raise KernelError("moe_gemm: one weight a pair")
-    out = torch.empty((slots, n), dtype=torch.float32 if pair_weight is not None else a.dtype, device=a.device)
+    if gated is not None and (pair_weight is not None or n % 2):
+        raise KernelError("moe_gemm: a gated product has an even number of rows and no pair weights")
+    epilogue = 2 + gate_act_code(gated) if gated is not None else (1 if pair_weight is not None else 0)
+    out = torch.empty((slots, n // 2 if gated is not None else n), dtype=torch.float32 if pair_weight is not None else a.dtype,
+                      device=a.device)
     check(load().fsie_moe_gemm(a.data_ptr(), weight.data_ptr(), out.data_ptr(), tiles.data_ptr(), tiles.shape[0],
-                               order.data_ptr(), int(gather_div), _ptr(pair_weight), n, k, 1 if pair_weight is not None else 0,
+                               order.data_ptr(), int(gather_div), _ptr(pair_weight), n, k, epilogue,
                                dtype_code(a.dtype), tile_rows, _stream()))
     return out
 

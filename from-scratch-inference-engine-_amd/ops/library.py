@@ -34,6 +34,9 @@ _SIGNATURES = {
     "fsie_random_fill": ([_P, c_int64, ctypes.c_uint64, c_int, c_float, _P], c_int),
     "fsie_swiglu": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_residual_add": ([_P, _P, c_int64, c_int, _P], c_int),
+    "fsie_round_to": ([_P, _P, c_int64, c_int, _P], c_int),
+    "fsie_scaled_sum": ([_P, c_float, _P, c_float, _P, c_int64, c_int, _P], c_int),
+    "fsie_pool_blocks": ([_P, _P, _P, c_int, c_int, _P, _P, _P, c_int, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_bias_add": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_sum_round": ([_P, c_int, _P, _P, c_int, c_int, _P], c_int),
     "fsie_rope_kv_write": ([_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
@@ -54,7 +57,7 @@ _SIGNATURES = {
     "fsie_fragment_order_size": ([c_int, c_int], c_int64),
     "fsie_fragment_order": ([_P, _P, c_int, c_int, _P], c_int),
     "fsie_attention_scalar": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
-                               c_int, c_int, c_float, c_int, _P, c_float, _P], c_int),
+                               c_int, c_int, c_float, c_int, _P, c_float, _P, _P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_attention_mfma": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
                              c_int, c_int, c_float, c_int, c_int, _P, c_float, _P], c_int),
     "fsie_attention_mfma_qkv_ok": ([c_int, c_int], c_int),
@@ -78,7 +81,7 @@ _SIGNATURES = {
                              ctypes.POINTER(c_int), ctypes.POINTER(c_int64)], c_int),
     "fsie_softcap": ([_P, c_int64, c_float, _P], c_int),
     "fsie_gla_scan": ([_P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, _P, _P, _P, c_int, c_int, c_int, c_int,
-                       c_float, c_float, c_int, c_int, _P], c_int),
+                       c_float, c_float, c_int, c_int, _P, _P], c_int),
     "fsie_latent_prep": ([_P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, _P, _P,
                           _P, _P, _P, c_int, c_int, c_int64, c_int, c_int, _P], c_int),
     "fsie_rope_pairs": ([_P, c_int64, c_int, c_int, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P, c_int, c_int,
@@ -91,7 +94,8 @@ _SIGNATURES = {
     "fsie_pair_embedding": ([_P, _P, c_int, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int64, c_int64,
                              c_float, _P], c_int),
     "fsie_attention_prep": ([_P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float,
-                             c_int, _P, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, _P], c_int),
+                             c_int, _P, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, c_int, c_float,
+                             _P], c_int),
     "fsie_gate_heads": ([_P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_group_rmsnorm": ([_P, _P, c_int, _P, c_int, c_float, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int,
                             _P], c_int),
@@ -102,7 +106,7 @@ _SIGNATURES = {
                          c_int, c_int, _P, _P, _P, _P, c_int, _P], c_int),
     "fsie_mlstm_scan_shape": ([c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int64)], c_int),
     "fsie_mlstm_out": ([_P, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_float, c_int, _P], c_int),
-    "fsie_moe_route": ([_P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_float, _P], c_int),
+    "fsie_moe_route": ([_P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_moe_group": ([_P, c_int, c_int, c_int, _P, _P, _P, c_int, _P], c_int),
     "fsie_moe_gemm": ([_P, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_moe_tile_rows": ([c_int, c_int], c_int),

@@ -9,8 +9,8 @@ import numpy as np
 import torch
 
 from .. import ops
-from ..cache.manager import PagedNeed
-from ..ops.functions import ATTN_ITEM_INTS, ATTN_KEEP_WALK, ATTN_MERGE_INTS
+from ..cache.manager import PagedNeed, PooledNeed
+from ..ops.functions import ATTN_ITEM_INTS, ATTN_KEEP_WALK, ATTN_MERGE_INTS, ATTN_POOL_WALK
 from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M
 from .base import Mixer, Norm, ParamDecl, Part, PositionEncoding, register_part
 from .linear import Linear
@@ -43,18 +43,52 @@ class AttentionPlanner:
     # Compute units to fill with the workgroups of small items; None: those of the device.
     compute_units: Optional[int] = None
 
-    def __init__(self, n_heads: int, n_kv: int, head_dim: int, window: Optional[int], keep_first: int = 0):
+    def __init__(self, n_heads: int, n_kv: int, head_dim: int, window: Optional[int], keep_first: int = 0,
+                 chunk: Optional[int] = None, pool: Optional[int] = None):
         """``keep_first`` (with a window): the first positions of a request stay visible to every later query.
         Items say so in their last field (``ATTN_ITEM_KEEP``); an item whose window has left those keys behind
         reads them first and then its own range (flag ``ATTN_KEEP_WALK``), and where a request's keys are split
-        over several items the kept keys are an item of their own that is merged with the rest."""
+        over several items the kept keys are an item of their own that is merged with the rest.
+
+        ``chunk`` (instead of a window): a query reads the keys of its own chunk of that many positions, counted
+        from the request's start, up to itself.  The kernels know nothing of it: a portion is cut where a chunk
+        ends, so all queries of an item share a chunk, and the item's range of keys starts where the chunk does.
+
+        ``pool`` (with a window): beside the window a query reads one pooled key and value for every block of
+        ``pool`` positions that lies wholly before its window.  Items carry the flag ``ATTN_POOL_WALK``; where a
+        request's keys are split over several items the pooled blocks are an item of their own.  The plan also
+        lists the blocks that the step completes (``pool_jobs``: request of the step, block), whose means the
+        mixer has computed before attention runs."""
+        if chunk and (window or keep_first):
+            raise ValueError("attention plan: chunks go without a window")
+        if pool and not window:
+            raise ValueError("attention plan: pooled blocks go with a window")
         self.n_heads, self.n_kv, self.head_dim, self.window = n_heads, n_kv, head_dim, window
         self.keep_first = int(keep_first) if window else 0
-        self.key = ("attention", n_heads, n_kv, head_dim, window, self.keep_first)
+        self.chunk, self.pool = (int(chunk) if chunk else None), (int(pool) if pool else None)
+        self.key = ("attention", n_heads, n_kv, head_dim, window, self.keep_first, self.chunk, self.pool)
         self._geometry = {}
+
+    def _portions(self, p: int, n: int):
+        """A request's n tokens from position p as (offset, tokens, position) runs whose queries share their first
+        key's rule: the portion itself, or with chunks its pieces between the chunks' ends."""
+        if not self.chunk or (p % self.chunk) + n <= self.chunk:
+            return [(0, n, p)]
+        runs, off = [], 0
+        while off < n:
+            here = min(n - off, self.chunk - (p + off) % self.chunk)
+            runs.append((off, here, p + off))
+            off += here
+        return runs
+
+    def _pooled_seen(self, last_pos: int) -> int:
+        """Pooled blocks that the query at ``last_pos`` reads."""
+        return max(0, last_pos - self.window + 1) // self.pool if self.pool else 0
 
     def _first_key(self, p: int):
         """(first key of the window of the query at position p, kept keys that lie before it)."""
+        if self.chunk:
+            return p // self.chunk * self.chunk, 0
         first = max(0, p - self.window + 1) if self.window else 0
         if self.keep_first and first <= self.keep_first:
             return 0, 0  # the kept keys and the window touch: one range, the mask does the rest
@@ -77,7 +111,7 @@ class AttentionPlanner:
 
     def uses_mfma(self, compute_dtype, page_size: int) -> bool:
         return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
-                and page_size % 4 == 0 and (not self.keep_first or self.mfma_keeps_first))
+                and page_size % 4 == 0 and (not self.keep_first or self.mfma_keeps_first) and not self.pool)
 
     mfma_keeps_first = True  # whether the matrix-core kernels read an item's kept first keys
 
@@ -93,10 +127,10 @@ class AttentionPlanner:
         """Keys that each small portion of the step reads."""
         keys = []
         for s in range(host.n_seqs):
-            n, p = host.q_lens[s], host.past_lens[s]
-            if n <= small_tokens:
-                first, kept = self._first_key(p)
-                keys.append(p + n - first + kept)
+            for _, n, p in self._portions(host.past_lens[s], host.q_lens[s]):
+                if n <= small_tokens:
+                    first, kept = self._first_key(p)
+                    keys.append(p + n - first + kept)
         return keys
 
     def split_keys(self, host, mfma: bool) -> int:
@@ -237,6 +271,7 @@ class AttentionPlanner:
             if mine > 1:
                 longest = max(longest, split_keys)
                 mine += 1 if kept else 0  # (the kept first keys are an item of their own)
+                mine += 1 if self._pooled_seen(host.past_lens[s] + host.q_lens[s] - 1) else 0  # (and the pooled blocks)
             elif kept:
                 longest = max(longest, keys + 32 * -(-kept // 32))
             n += mine
@@ -262,48 +297,59 @@ class AttentionPlanner:
         small, merges = [], []
         large_runs = []  # per long portion: its tiles as rows of an array (a prompt of thousands of tokens has hundreds)
         n_partial = 0
+        pool_flag = ATTN_POOL_WALK if self.pool else 0
+        pool_jobs = []
         for s in range(host.n_seqs):
-            n, p, row0 = host.q_lens[s], host.past_lens[s], host.q_starts[s]
-            first_key, kept = self._first_key(p)
-            keep = self.keep_first
-            total = p + n
-            n_splits = self._items_of(total - first_key, split_keys, most) if split_keys is not None else 1
-            if n <= small_tokens and n_splits > 1:
-                base = n_partial
-                if kept:
-                    small.append((s, row0, n, p, 0, kept, base, keep))
-                    base += n
-                for i in range(n_splits):
-                    kb = first_key + i * split_keys
-                    small.append((s, row0, n, p, kb, total if i == n_splits - 1 else kb + split_keys, base + i * n, keep))
-                n_splits += 1 if kept else 0
-                for t in range(n):
-                    merges.append((row0 + t, n_partial + t, n_splits, n))
-                n_partial += n_splits * n
-            elif n <= small_tokens:
-                small.append((s, row0, n, p, first_key, total, -1, keep | ATTN_KEEP_WALK if keep else 0))
-            else:
-                # (the short tile that a long portion may end with stays with the portion's other tiles:
-                # as a small item it would walk all the portion's keys in one workgroup a kv head, alone
-                # on the device, while as the last of a group of four it shares their blocks of keys)
-                t0 = np.arange(0, n, large_tokens, dtype=np.int64)
-                run = np.empty((t0.shape[0], ATTN_ITEM_INTS), dtype=np.int64)
-                pos0 = p + t0
-                run[:, 0] = s
-                run[:, 1] = row0 + t0
-                run[:, 2] = np.minimum(large_tokens, n - t0)
-                run[:, 3] = pos0
-                run[:, 4] = np.maximum(0, pos0 - self.window + 1) if self.window else 0
-                if self.keep_first:
-                    run[:, 4] = np.where(run[:, 4] <= self.keep_first, 0, run[:, 4])
-                run[:, 5] = pos0 + run[:, 2]
-                run[:, 6] = -1
-                run[:, 7] = self.keep_first | ATTN_KEEP_WALK if self.keep_first else 0
-                large_runs.append(run)
+            if self.pool:
+                # the blocks whose last position this step brings: their means are made before attention runs
+                p_all, n_all = host.past_lens[s], host.q_lens[s]
+                pool_jobs += [(s, b) for b in range(p_all // self.pool, (p_all + n_all) // self.pool)]
+            for off, n, p in self._portions(host.past_lens[s], host.q_lens[s]):
+                row0 = host.q_starts[s] + off
+                first_key, kept = self._first_key(p)
+                keep = self.keep_first
+                total = p + n
+                n_splits = self._items_of(total - first_key, split_keys, most) if split_keys is not None else 1
+                if n <= small_tokens and n_splits > 1:
+                    base = n_partial
+                    if kept:
+                        small.append((s, row0, n, p, 0, kept, base, keep))
+                        base += n
+                    pooled = self._pooled_seen(total - 1) > 0
+                    if pooled:  # the pooled blocks: an item with no keys of its own
+                        small.append((s, row0, n, p, 0, 0, base, keep | pool_flag))
+                        base += n
+                    for i in range(n_splits):
+                        kb = first_key + i * split_keys
+                        small.append((s, row0, n, p, kb, total if i == n_splits - 1 else kb + split_keys, base + i * n, keep))
+                    n_splits += (1 if kept else 0) + (1 if pooled else 0)
+                    for t in range(n):
+                        merges.append((row0 + t, n_partial + t, n_splits, n))
+                    n_partial += n_splits * n
+                elif n <= small_tokens:
+                    small.append((s, row0, n, p, first_key, total, -1, (keep | ATTN_KEEP_WALK if keep else 0) | pool_flag))
+                else:
+                    # (the short tile that a long portion may end with stays with the portion's other tiles:
+                    # as a small item it would walk all the portion's keys in one workgroup a kv head, alone
+                    # on the device, while as the last of a group of four it shares their blocks of keys)
+                    t0 = np.arange(0, n, large_tokens, dtype=np.int64)
+                    run = np.empty((t0.shape[0], ATTN_ITEM_INTS), dtype=np.int64)
+                    pos0 = p + t0
+                    run[:, 0] = s
+                    run[:, 1] = row0 + t0
+                    run[:, 2] = np.minimum(large_tokens, n - t0)
+                    run[:, 3] = pos0
+                    run[:, 4] = np.maximum(0, pos0 - self.window + 1) if self.window else (first_key if self.chunk else 0)
+                    if self.keep_first:
+                        run[:, 4] = np.where(run[:, 4] <= self.keep_first, 0, run[:, 4])
+                    run[:, 5] = pos0 + run[:, 2]
+                    run[:, 6] = -1
+                    run[:, 7] = (self.keep_first | ATTN_KEEP_WALK if self.keep_first else 0) | pool_flag
+                    large_runs.append(run)
         large = np.concatenate(large_runs) if large_runs else np.zeros((0, ATTN_ITEM_INTS), dtype=np.int64)
         waves = 1
         if mfma and small:
-            waves = self._waves_for(max(it[5] - it[4] + (32 * -(-min(it[7] & ~ATTN_KEEP_WALK, it[4]) // 32)
+            waves = self._waves_for(max(it[5] - it[4] + (32 * -(-min(it[7] & ~(ATTN_KEEP_WALK | ATTN_POOL_WALK), it[4]) // 32)
                                                             if it[7] & ATTN_KEEP_WALK else 0) for it in small),
                                     ops.attention_mfma_max_waves(self.head_dim))
         if padded:
@@ -341,7 +387,15 @@ class AttentionPlanner:
             large = np.concatenate([large[~is_long], large[is_long]])
             n_long = int(is_long.sum())
         small_items = np.asarray(small, dtype=np.int64).reshape(-1, ATTN_ITEM_INTS)
+        extra = {}
+        if self.pool:
+            if padded:  # (a step of single tokens completes at most a block a request)
+                if len(pool_jobs) > host.n_seqs:
+                    raise RuntimeError("attention plan: more completed blocks than the captured graph has room for")
+                pool_jobs += [(-1, 0)] * (host.n_seqs - len(pool_jobs))
+            extra = {"pool_jobs": np.asarray(pool_jobs, dtype=np.int32).reshape(-1, 2), "n_pool_jobs": len(pool_jobs)}
         return {
+            **extra,
             "items": np.concatenate([small_items, large]).astype(np.int32),
             "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
             "groups": groups.astype(np.int32), "n_groups": len(groups),
@@ -353,15 +407,18 @@ class AttentionPlanner:
 
 def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n_kv: int, head_dim: int,
                     window: Optional[int], scale: float, n_tokens: int, sinks: Optional[torch.Tensor] = None,
-                    share_keys: bool = True, softcap: Optional[float] = None) -> torch.Tensor:
+                    share_keys: bool = True, softcap: Optional[float] = None, pooled=None) -> torch.Tensor:
     """Causal attention of a step's queries over the paged cache, by the work items of ``plan`` (an
     ``AttentionPlanner``'s): [n_tokens, n_heads * head_dim] in the queries' type.  ``q``: rows of ``q_stride``
     values whose first n_heads * head_dim are the heads' queries; the keys and values of the step's own
     tokens are in the cache already.  ``sinks`` (float32 [n_heads] or None): a term exp(sinks[h]) more in the
     denominator of head h's softmax.  ``softcap`` (a positive number or None): the scaled scores become
-    softcap * tanh(score / softcap) before the mask and the softmax.  Every mixer whose cache is pages of keys and
-    values calls this."""
+    softcap * tanh(score / softcap) before the mask and the softmax.  ``pooled`` = (k_pool, v_pool, block_tables,
+    block_tokens): the pools of pooled blocks that items flagged ``ATTN_POOL_WALK`` read beside their keys (a planner
+    with ``pool``).  Every mixer whose cache is pages of keys and values calls this."""
     cap = float(softcap or 0.0)
+    if pooled is not None and plan.mfma:
+        raise RuntimeError("attention: pooled blocks are read by the float32-arithmetic kernel alone")
     out = torch.empty((n_tokens, n_heads * head_dim), dtype=q.dtype, device=q.device)
     partials = None
     if plan.n_partial:
@@ -384,7 +441,7 @@ def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n
                                waves=4, sinks=sinks, softcap=cap)
     else:
         ops.attention_scalar(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
-                             plan.n_small + plan.n_large, out, *args, sinks=sinks, softcap=cap)
+                             plan.n_small + plan.n_large, out, *args, sinks=sinks, softcap=cap, pooled=pooled)
     if plan.n_merges:
         ops.attention_merge(partials, plan.merges, plan.n_merges, out, n_heads, head_dim, sinks=sinks)
     return out
@@ -410,6 +467,17 @@ class GQAttention(Mixer):
     order, norm then rotation, gives the same head as rotation then norm).  ``head_temperature=True`` (with
     ``unit_norm_eps``): a number per query head (parameter ``temperature``) multiplies its scores.  ``softcap``: the
     scaled scores become softcap * tanh(score / softcap).
+    ``interleaved_pairs=True``: the encoding rotates neighbours (2i, 2i + 1) of the checkpoint's heads; the rows of the
+    q and k projections and the head norms' weights are reordered once, when the weights are loaded (even values of the
+    rotated part first, then the odd ones), so that the rotation is that of the pairs (i, i + rotary_dim / 2): the scores
+    do not change when q and k are reordered alike, and nothing else reads them.  ``value_unit_norm_eps``: every kv
+    head's values are divided by their root mean square (eps inside the root, no weight) before they are cached.
+    ``unit_sink=True``: one is added to the softmax's denominator (a sink whose score is 0, without a value).
+    ``chunk`` (instead of a window): a query reads the keys of its own chunk of that many positions, counted from the
+    request's start.  ``pool`` (with a window): beside the window a query reads the mean key and mean value of every
+    block of ``pool`` positions that lies wholly before its window; the means are kept in pages of their own (an entry a
+    block, a second cache need) and made by a kernel from the cached keys and values when a block's last position
+    arrives.  ``fused_prep=True`` takes the one-kernel path below also where none of its reasons holds.
     With any of gate, mixed values, another value size or the unit norm, what stands between projection and attention is one kernel
     (``ops.attention_prep``: head norms, rotation of the first ``rotary_dim`` values from the step's table, value
     mixing, gates, cache write) and one after it (``ops.gate_heads``).
@@ -440,7 +508,9 @@ class GQAttention(Mixer):
                  k_norm: Optional[Norm] = None, sink: bool = False, keep_first: int = 0, scale: Optional[float] = None,
                  value_dim: Optional[int] = None, gate: bool = False, value_mix: Optional[str] = None,
                  o_bias: bool = False, unit_norm_eps: Optional[float] = None, head_temperature: bool = False,
-                 softcap: Optional[float] = None):
+                 softcap: Optional[float] = None, interleaved_pairs: bool = False,
+                 value_unit_norm_eps: Optional[float] = None, unit_sink: bool = False, chunk: Optional[int] = None,
+                 pool: Optional[int] = None, fused_prep: bool = False):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: heads {n_heads} must be a multiple of kv heads {n_kv_heads}")
         self.value_dim = head_dim if value_dim is None else int(value_dim)
@@ -468,7 +538,19 @@ class GQAttention(Mixer):
         self.softcap = None if softcap is None else float(softcap)
         self.temperature: Optional[torch.Tensor] = None
         self._unit_q = self._unit_k = None  # the unit norm's weights: the temperature (or 1) for q, 1 for k
-        self.prepared = self.has_gate or value_mix is not None or self.value_dim != head_dim or self.unit_norm_eps is not None
+        self.interleaved_pairs = bool(interleaved_pairs)
+        self._reordered = False
+        self.value_unit_norm_eps = None if value_unit_norm_eps is None else float(value_unit_norm_eps)
+        self.unit_sink = bool(unit_sink)
+        if unit_sink and sink:
+            raise ValueError("attention: a learned sink or the sink of score 0, not both")
+        if chunk is not None and (chunk < 1 or window or keep_first):
+            raise ValueError("attention: a chunk is a positive number of positions and goes without a window")
+        if pool is not None and (pool < 1 or not window or keep_first):
+            raise ValueError("attention: pooled blocks are a positive number of positions and go with a plain window")
+        self.chunk, self.pool = chunk, pool
+        self.prepared = (self.has_gate or value_mix is not None or self.value_dim != head_dim or self.unit_norm_eps is not None
+                         or self.value_unit_norm_eps is not None or pool is not None or bool(fused_prep) or self.interleaved_pairs)
         if self.prepared:
             if position.rotates and getattr(position, "layout", None) != "half":
                 raise ValueError("attention: with a gate, mixed values or values of another size the position encoding "
@@ -521,6 +603,22 @@ class GQAttention(Mixer):
         bias = self.qkv.bias
         if self.has_gate and bias is not None and bias.shape[0] == self.qkv.out_features - self.n_heads:
             self.qkv.bias = torch.cat([bias, torch.zeros((self.n_heads,), dtype=bias.dtype, device=bias.device)])
+        if self.interleaved_pairs and not self._reordered and self.rot_pairs:
+            # neighbours (2i, 2i + 1) of the rotated part become the pairs (i, i + pairs): q and k rows and the head
+            # norms' weights alike
+            hd, rot = self.head_dim, 2 * self.rot_pairs
+            order = torch.cat([torch.arange(0, rot, 2), torch.arange(1, rot, 2), torch.arange(rot, hd)]).to(device)
+            heads = torch.arange(self.n_heads + self.n_kv, device=device)
+            rows = torch.arange(self.qkv.out_features, device=device)
+            rows[:self.q_dim + self.kv_dim] = (heads[:, None] * hd + order[None, :]).reshape(-1)
+            self.qkv.weight = self.qkv.weight[rows].contiguous()
+            if self.qkv.bias is not None:
+                self.qkv.bias = self.qkv.bias[rows[:self.qkv.bias.shape[0]]].contiguous()
+            for norm in {id(n): n for n in (self.q_norm, self.k_norm) if n is not None}.values():
+                norm.weight = norm.weight[order].contiguous()
+            self._reordered = True
+        if self.unit_sink:
+            self.sink = torch.zeros((self.n_heads,), dtype=torch.float32, device=device)
         if self.unit_norm_eps is not None:
             ones = torch.ones((self.n_heads, self.head_dim), dtype=torch.float32, device=device)
             self._unit_k = ones[0].contiguous()
@@ -533,12 +631,20 @@ class GQAttention(Mixer):
         return self.qkv.drop_copy() + self.o.drop_copy()
 
     # cache and plan ---------------------------------------------------------------------
-    def cache_need(self) -> PagedNeed:
+    def cache_need(self):
+        if self.chunk:
+            # (a query reads no key before its chunk's start: the pages a chunk's length back go to the pool again)
+            return PagedNeed(self.n_kv, self.padded, self.chunk, 0)
+        if self.pool:
+            # keys and values of the window (a block's positions stay until its means are made), and the pooled blocks
+            return {"tokens": PagedNeed(self.n_kv, self.padded, max(self.window, self.pool), 0),
+                    "blocks": PooledNeed(self.n_kv, self.padded, None, 0, self.pool)}
         return PagedNeed(self.n_kv, self.padded, self.window, self.keep_first if self.window else 0)
 
     def planner(self) -> AttentionPlanner:
         if self._planner is None:
-            self._planner = AttentionPlanner(self.n_heads, self.n_kv, self.padded, self.window, self.keep_first)
+            self._planner = AttentionPlanner(self.n_heads, self.n_kv, self.padded, self.window, self.keep_first,
+                                             chunk=self.chunk, pool=self.pool)
         return self._planner
 
     # compute ----------------------------------------------------------------------------
@@ -616,6 +722,9 @@ class GQAttention(Mixer):
         """Gate, mixed values or values of another size than the keys: the fused projection, one kernel for all
         that stands between it and attention, attention over heads of ``padded`` values, the gate."""
         nh, nkv, hd, vd, pd = self.n_heads, self.n_kv, self.head_dim, self.value_dim, self.padded
+        blocks = None
+        if self.pool:
+            cache, blocks = cache["tokens"], cache["blocks"]
         proj = self.qkv(x)
         k_off, v_off = self.q_dim, self.q_dim + self.kv_dim
         g_off = v_off + self.v_dim
@@ -639,9 +748,16 @@ class GQAttention(Mixer):
         q, gate = ops.attention_prep(proj, 0, k_off, v_off, g_off, nh, nkv, hd, vd, pd, q_weight, k_weight, eps,
                                      self.rot_pairs, table, self.has_gate,
                                      v_other=other, v_other_stride=other_stride,
-                                     mix=self.value_mix_weight if other is not None else None, **store)
+                                     mix=self.value_mix_weight if other is not None else None,
+                                     v_unit_norm_eps=self.value_unit_norm_eps, **store)
+        pooled = None
+        if blocks is not None:
+            if cache.writes and plan.n_pool_jobs:
+                ops.pool_blocks(cache.k_pool, cache.v_pool, cache.block_tables, blocks.k_pool, blocks.v_pool,
+                                blocks.block_tables, plan.pool_jobs, plan.n_pool_jobs, self.pool)
+            pooled = (blocks.k_pool, blocks.v_pool, blocks.block_tables, self.pool)
         out = paged_attention(q, nh * pd, cache, plan, nh, nkv, pd, self.window, self.scale, x.shape[0], sinks=self.sink,
-                              share_keys=self.share_keys, softcap=self.softcap)
+                              share_keys=self.share_keys, softcap=self.softcap, pooled=pooled)
         if gate is not None or pd != vd:
             out = ops.gate_heads(out, pd, vd, nh, gate)
         return self.o.for_residual(out, ctx)

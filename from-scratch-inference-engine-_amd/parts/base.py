@@ -34,7 +34,8 @@ class ParamDecl:
     """A parameter of a part.  ``storage``: 'matrix' (compute dtype), 'vector' (float32) or
     'int_table' (int32).  ``init`` names the random-weights distribution.  ``layout`` says how
     several checkpoint tensors make up the parameter: 'concat' (one after the other along dim
-    0) or 'interleave' (row i of every source in turn: a0, b0, a1, b1, ...)."""
+    0), 'interleave' (row i of every source in turn: a0, b0, a1, b1, ...) or 'interleave_pairs' (the sources two by
+    two, each pair interleaved, the pairs one after the other: an expert's gate and up rows in turn, expert by expert)."""
 
     shape: Tuple[int, ...]
     storage: str = "matrix"

@@ -60,6 +60,36 @@ class SandwichNormBlock(Block):
             hidden.delta, hidden.delta_norm = self.ffn.forward(x, ctx), self.ffn_post_norm
 
 
+@register_part("block", "branch_norm")
+class BranchNormBlock(Block):
+    """Norms on the sublayers' outputs only: x += post1(mixer(x)); x += post2(ffn(x)).  The sublayers read the stream
+    itself (``reader``: a norm part that returns the stream as it is, ``stream``).  A sublayer's output stays pending
+    with its norm; whoever reads the stream next (this block's reader, the next block's, the model's last norm) runs
+    that norm and the sum in its own pass.  ``ffn=None``: the layer has no feed-forward."""
+
+    graph_safe = True
+
+    def __init__(self, reader: Norm, mixer: Mixer, mixer_post_norm: Norm, ffn: Optional[FeedForward] = None,
+                 ffn_post_norm: Optional[Norm] = None):
+        if (ffn is None) != (ffn_post_norm is None):
+            raise ValueError("branch_norm block: a feed-forward comes with the norm of its output, or neither")
+        self.reader, self.mixer, self.mixer_post_norm = reader, mixer, mixer_post_norm
+        self.ffn, self.ffn_post_norm = ffn, ffn_post_norm
+
+    def sub_parts(self) -> Dict[str, Part]:
+        parts = {"reader": self.reader, "mixer": self.mixer, "mixer_post_norm": self.mixer_post_norm}
+        if self.ffn is not None:
+            parts.update(ffn=self.ffn, ffn_post_norm=self.ffn_post_norm)
+        return parts
+
+    def forward(self, hidden: HiddenState, ctx, cache) -> None:
+        x = self.reader(hidden, ctx.compute_dtype)
+        hidden.delta, hidden.delta_norm = self.mixer.forward(x, ctx, cache), self.mixer_post_norm
+        if self.ffn is not None:
+            x = self.reader(hidden, ctx.compute_dtype)
+            hidden.delta, hidden.delta_norm = self.ffn.forward(x, ctx), self.ffn_post_norm
+
+
 @register_part("block", "parallel")
 class ParallelBlock(Block):
     """Mixer and feed-forward side by side: x += mixer(norm1(x)) + ffn(norm2(x)), both norms of the same x.  The two

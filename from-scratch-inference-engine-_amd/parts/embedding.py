@@ -13,21 +13,27 @@ from .linear import Linear
 
 class TokenEmbedding(Part):
     """x[t] = table[ids[t]] (src/model/nn.cpp:90-108, which does not scale) times ``scale``, written as
-    the float32 residual stream."""
+    the float32 residual stream.  ``norm`` (a norm part as wide as the stream, or None): the rows go through it, in
+    float32, before they become the stream."""
 
     kind = "embedding"
     graph_safe = True  # reads the step's token ids from the device
 
-    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, norm=None):
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.scale = float(scale)
+        self.norm = norm
         self.weight = None
+
+    def sub_parts(self):
+        return {} if self.norm is None else {"norm": self.norm}
 
     def param_decls(self) -> Dict[str, ParamDecl]:
         return {"weight": ParamDecl((self.vocab_size, self.hidden_size))}
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return ops.embedding(self.weight, ids, scale=self.scale)
+        x = ops.embedding(self.weight, ids, scale=self.scale)
+        return x if self.norm is None else self.norm.plain(x, out=x)
 
     def cache_need(self):
         """What the embedding keeps for a request between steps (a need of ``cache.needs``), or None."""

@@ -16,7 +16,7 @@ from .linear import Linear
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
     """down(act(gate(x)) * up(x)), no biases, act = SiLU (src/model/model.cpp:134-138) unless ``activation``
-    names another one the kernels know ("gelu_tanh").  gate and up are one
+    names another one the kernels know ("gelu_tanh", "relu").  gate and up are one
     matrix [2I, H] with their rows interleaved (gate_0, up_0, gate_1, up_1, ...): x is read once,
     and the lane that holds gate_j also holds up_j, so that for a few rows (decoding) SiLU*up
     happens in the product's epilogue and the [T, 2I] intermediate never reaches memory."""
@@ -77,7 +77,7 @@ class SwiGLU(FeedForward):
             act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.weight, act=self.activation)
         elif x.dtype == torch.bfloat16 and m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 8 == 0:
             act = ops.gemm_mfma_skinny(x, self.gate_up.weight,
-                                       epilogue="swiglu" if self.activation == "silu" else "geglu_tanh")
+                                       epilogue={"silu": "swiglu", "gelu_tanh": "geglu_tanh", "relu": "reglu"}[self.activation])
         else:
             act = ops.swiglu(self.gate_up(x), act=self.activation)
         return self.down.for_residual(act, ctx)

@@ -172,3 +172,38 @@ class GroupRMSNorm(Norm):
         d1, d2, scale = self._take(hidden, False)
         return ops.group_rmsnorm(hidden.residual, self.weight, self.eps, self.groups, out_dtype, delta=d1, delta2=d2,
                                  delta_scale=scale, rows=rows)
+
+
+@register_part("norm", "stream")
+class StreamReader(Norm):
+    """No norm at all: the stream itself, x = residual + pending delta, in the type asked for.  It stands where a
+    layer's sublayers read the stream as it is and only their outputs are normed: the pending delta then comes with
+    a norm of its own (``HiddenState.delta_norm``, an ``RMSNorm``), and that norm, the float32 sum and the rounding of
+    the result are one kernel."""
+
+    adds_partial_sums = True
+    graph_safe = True
+
+    def __init__(self, hidden_size: int):
+        self.hidden_size = hidden_size
+
+    @staticmethod
+    def _pending(hidden: HiddenState):
+        _no_second_delta(hidden, "stream")
+        delta, post = hidden.delta, hidden.delta_norm
+        if delta is not None and post is None:
+            raise RuntimeError("stream: a pending delta without a norm of its own is not taken (a pre-norm block came before)")
+        return delta, post
+
+    def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
+        delta, post = self._pending(hidden)
+        hidden.delta = hidden.delta_norm = None
+        if delta is None:
+            return hidden.residual if out_dtype == torch.float32 else ops.round_to(hidden.residual, out_dtype)
+        return ops.sandwich_norm(hidden.residual, delta, post.weight, post.eps, None, 0.0, out_dtype, write_back=True)
+
+    def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        delta, post = self._pending(hidden)
+        if delta is None:
+            raise RuntimeError("stream: chosen rows of a stream without a pending delta are not offered")
+        return ops.sandwich_norm(hidden.residual, delta, post.weight, post.eps, None, 0.0, out_dtype, rows=rows)

@@ -26,12 +26,16 @@ class RotaryEncoding(PositionEncoding):
     hi = min(ceil(dim(slow)), rotary_dim - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i
     turns at f_i / factor * ramp_i + f_i * (1 - ramp_i) (fast pairs stay, slow pairs are divided by the factor,
     a ramp between), and every cosine and sine is multiplied by 0.1 * ln(factor) + 1.  That factor only exists
-    in the table: ``rotate`` refuses where it would have to compute the angles itself."""
+    in the table: ``rotate`` refuses where it would have to compute the angles itself.
+
+    ``bands`` = (factor, low, high, original) rescales by wavelength instead: with l_i = 2 pi / f_i, a pair whose
+    wavelength is below original / high keeps f_i, one above original / low turns at f_i / factor, and between the two
+    s = (original / l_i - low) / (high - low) blends them, (1 - s) f_i / factor + s f_i."""
 
     graph_safe = True
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, layout: str = "half",
-                 stretch: Optional[tuple] = None):
+                 stretch: Optional[tuple] = None, bands: Optional[tuple] = None):
         if layout not in ("half", "interleaved"):
             raise ValueError(f"rope: unknown layout '{layout}' (half or interleaved)")
         self.layout = layout
@@ -42,6 +46,12 @@ class RotaryEncoding(PositionEncoding):
             raise ValueError(f"rope: rotary_dim {self.rotary_dim} must be even and within head_dim {head_dim}")
         self.inv_freq = None
         self.magnitude = 1.0
+        self.bands = None
+        if bands is not None:
+            factor, low, high, original = (float(v) for v in bands)
+            if stretch is not None or not (factor > 0 and original > 0 and 0 < low < high):
+                raise ValueError(f"rope: bands {bands} need a positive factor and original and 0 < low < high (and no stretch)")
+            self.bands = (factor, low, high, original)
         self.stretch = None
         if stretch is not None:
             factor, original, fast, slow = (float(v) for v in stretch)
@@ -55,6 +65,12 @@ class RotaryEncoding(PositionEncoding):
         dims = self.rotary_dim
         i = np.arange(dims // 2, dtype=np.float64)
         freq = np.power(np.float64(self.theta), -2.0 * i / dims)
+        if self.bands is not None:
+            factor, low, high, original = self.bands
+            wavelength = 2.0 * math.pi / freq
+            blend = (original / wavelength - low) / (high - low)
+            mixed = (1.0 - blend) * freq / factor + blend * freq
+            return np.where(wavelength < original / high, freq, np.where(wavelength > original / low, freq / factor, mixed))
         if self.stretch is None:
             return freq
         factor, original, fast, slow = self.stretch
@@ -73,7 +89,7 @@ class RotaryEncoding(PositionEncoding):
     def table(self, ctx) -> torch.Tensor:
         """The cosines and sines of this step's positions: the same in every layer, made by the
         first one that asks."""
-        key = ("rope cos/sin", self.theta, self.rotary_dim, self.stretch)
+        key = ("rope cos/sin", self.theta, self.rotary_dim, self.stretch, self.bands)
         table = ctx.memo.get(key)
         if table is None:
             table = ctx.memo[key] = ops.rope_table(ctx.positions, self.inv_freq, self.magnitude)

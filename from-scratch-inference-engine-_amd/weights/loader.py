@@ -47,13 +47,14 @@ class TensorSpec:
 @dataclass
 class ParamBinding:
     """Parameter ``attr`` of ``owner`` = the sources joined along dim 0 ('concat': one after the
-    other; 'interleave': row i of every source in turn), kept as ``storage``."""
+    other; 'interleave': row i of every source in turn; 'interleave_pairs': the sources two by two, row i of the
+    pair's first and of its second in turn, the pairs one after the other), kept as ``storage``."""
 
     owner: Any
     attr: str
     sources: Sequence[TensorSpec]
     storage: str = "matrix"  # matrix | vector | int_table
-    layout: str = "concat"   # concat | interleave
+    layout: str = "concat"   # concat | interleave | interleave_pairs
 
 
 def expected_tensors(bindings: Sequence[ParamBinding]) -> Dict[str, TensorSpec]:
@@ -155,6 +156,11 @@ def fill_parts(bindings: Sequence[ParamBinding], get_tensor, compute_dtype: torc
                 if any(p.shape != pieces[0].shape for p in pieces):
                     raise WeightsError(f"{b.attr}: interleaved sources must have equal shapes")
                 value = torch.stack(pieces, dim=1).reshape(-1, *pieces[0].shape[1:])
+            elif b.layout == "interleave_pairs":
+                if len(pieces) % 2 or any(p.shape != pieces[0].shape for p in pieces):
+                    raise WeightsError(f"{b.attr}: sources interleaved in pairs must be an even number of equal shapes")
+                value = torch.cat([torch.stack(pieces[i:i + 2], dim=1).reshape(-1, *pieces[0].shape[1:])
+                                   for i in range(0, len(pieces), 2)], dim=0)
             elif b.layout == "concat":
                 value = torch.cat(pieces, dim=0)
             else:
