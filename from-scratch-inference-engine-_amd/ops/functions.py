@@ -802,6 +802,8 @@ def sandwich_norm(residual: torch.Tensor, delta: torch.Tensor, post_weight: torc
         _need(weight, "sandwich_norm weight", dtype=torch.float32, shape=(h,))
     _need(post_weight, "sandwich_norm post weight", dtype=torch.float32, shape=(h,))
     n_parts = 0
+    if delta.ndim == 2 and delta.dtype == torch.float32 and out_dtype != torch.float32:
+        delta = delta.unsqueeze(0)  # a float32 delta beside 16-bit activations (the experts' sum): one plane of sums
     if delta.ndim == 3:
         n_parts = delta.shape[0]
         _need(delta, "sandwich_norm delta parts", dtype=torch.float32, shape=(n_parts, t, h))
