@@ -54,6 +54,11 @@ def rms_norm(x, w, eps):
     return unit_rms(x, eps) * w
 
 
+def value_norm(v, eps):
+    """Every head's values divided by their root mean square (no weight)."""
+    return unit_rms(v, eps)
+
+
 def silu(z):
     return z / (1.0 + np.exp(-z))
 
@@ -194,7 +199,7 @@ def chunked_mixer(h, w, p, m, eps):
     heads, kv, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = rms_norm((h @ w[p + "q"].T).reshape(t, heads, d), w[p + "q.norm"], eps)
     k = rms_norm((h @ w[p + "k"].T).reshape(t, kv, d), w[p + "k.norm"], eps)
-    v = unit_rms((h @ w[p + "v"].T).reshape(t, kv, e), eps)
+    v = value_norm((h @ w[p + "v"].T).reshape(t, kv, e), eps)
     o = chunk_attention(q, k, v, m["scale"], m["mask"]["size"])
     return o.reshape(t, heads * e) @ w[p + "o"].T
 
