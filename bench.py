@@ -284,12 +284,33 @@ def fiterax_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
             "embedding": {"scale": 10.0}, "residual_mult": 0.25, "canon": {"taps": 4}, "layers": out}
 
 
-DESIGN_SHAPES = {"gilozen": gilozen_shape, "botulorn": botulorn_shape, "fiterax": fiterax_shape}
+def mafosun_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Mafosun configuration of real layer sizes: layers of chunked attention beside retention and layers of attention
+    over a window of 1,024 positions with pooled blocks of 64 in turn, a dense feed-forward and eight routed experts in
+    two groups (two a token, from the best group) in turn; an expert has gate, up and down of ff / 8, so a token's two
+    experts are a quarter of the dense feed-forward's arithmetic."""
+    heads = width // 128
+    bands = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
+    gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
+           "mask": {"size": 1024, "pool": 64}, "rot": {"base": 500000.0, "dims": 64, "scaling": bands}}
+    pair = {"left": {"heads": heads // 2, "kv_heads": max(1, width // 1024), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "mask": {"size": 512}},
+            "right": {"heads": width // 256, "dim": 128, "vdim": 128, "rot": {"base": 500000.0, "dims": 128},
+                      "decay": [1.0 - 2.0 ** -(5 + i % 6) for i in range(width // 256)]},
+            "left_scale": 1.2, "right_scale": 0.5}
+    dense = {"kind": "dense", "ff": ff}
+    routed = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 8, "top": 2, "groups": {"count": 2, "keep": 1}}}
+    out = [{"type": "parallel" if i % 2 == 0 else "attention", "mixer": dict(pair if i % 2 == 0 else gqa),
+            "mlp": dict(dense if i % 4 < 2 else routed)} for i in range(layers)]
+    return {"architecture": "Mafosun", "width": width, "vocab": vocab, "norm": {"eps": 1e-5}, "layers": out}
+
+
+DESIGN_SHAPES = {"gilozen": gilozen_shape, "botulorn": botulorn_shape, "fiterax": fiterax_shape, "mafosun": mafosun_shape}
 DESIGN_SIZES = {"2048": (2048, 8192, 9, 32000), "4096": (4096, 14336, 9, 32000)}  # width, ff, layers, vocab
 
 
 def design_comparison(args) -> int:
-    """--workload gilozen | botulorn | fiterax: prefill (one prompt of 2,048 tokens in one step) and decode (batches of 8 and 64 at a
+    """--workload gilozen | botulorn | fiterax | mafosun: prefill (one prompt of 2,048 tokens in one step) and decode (batches of 8 and 64 at a
     context of 512, from captured graphs) of the named design at two real layer sizes with random weights, beside a Qwen2
     model of the same width, feed-forward, layers and vocabulary (grouped-query attention, 128 values a head, four
     query heads a key/value head) through the same step function.  One JSON line."""
@@ -374,14 +395,14 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
     ap.add_argument("--no-streamed-copies", action="store_true",
                     help="do not keep the large weights a second time in the order of the matrix instruction's fragments")
-    ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen | botulorn | fiterax: widths to run (2048, 4096)")
-    ap.add_argument("--design-batches", default="8,64", help="--workload gilozen | botulorn | fiterax: decode batches to time (at most 64)")
-    ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen | botulorn | fiterax: what to time (for a trace of one phase)")
-    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen", "botulorn", "fiterax"], default="decode",
+    ap.add_argument("--design-sizes", default="2048,4096", help="--workload gilozen | botulorn | fiterax | mafosun: widths to run (2048, 4096)")
+    ap.add_argument("--design-batches", default="8,64", help="--workload gilozen | botulorn | fiterax | mafosun: decode batches to time (at most 64)")
+    ap.add_argument("--design-phases", default="prefill,decode", help="--workload gilozen | botulorn | fiterax | mafosun: what to time (for a trace of one phase)")
+    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill", "gilozen", "botulorn", "fiterax", "mafosun"], default="decode",
                     help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "
                          "--outputs tokens each, through the scheduler (made for --shape 14b).  "
                          "long-prefill: one prompt of --prefill-tokens tokens in portions of the token budget "
-                         "(made for --shape 32b).  gilozen, botulorn, fiterax: that design beside Qwen2 at equal layer sizes")
+                         "(made for --shape 32b).  gilozen, botulorn, fiterax, mafosun: that design beside Qwen2 at equal layer sizes")
     ap.add_argument("--requests", type=int, default=32)
     ap.add_argument("--min-prompt", type=int, default=128)
     ap.add_argument("--max-prompt", type=int, default=4096)

@@ -298,13 +298,19 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
                              float* state, const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens,
                              float* prep, float* out, float* chunk_work, int max_chunks, int heads, int dim, int vdim,
                              float q_scale, float inv_tau, int n_slots, int dtype, const float* head_decay,
-                             hipStream_t stream) {
+                             const void* qk, int64_t qk_stride, hipStream_t stream) {
+    // q and k may live in rows of their own (qk, rows qk_stride apart, the same column offsets): a caller that has
+    // turned them by the positions without touching the projection
+    const void* qk_rows = qk ? qk : proj;
+    const int64_t qk_step = qk ? qk_stride : proj_stride;
+    FSIE_REQUIRE(!qk || (q_off + heads * dim <= qk_stride && k_off + heads * dim <= qk_stride),
+                 "gla_scan: the q and k columns do not fit a row of %lld", static_cast<long long>(qk_stride));
     FSIE_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && heads > 0 && dim > 0 && vdim > 0 && n_slots > 0, "gla_scan: bad sizes");
     FSIE_REQUIRE(dim <= 256, "gla_scan: %d key channels a head are more than the kernel takes (256)", dim);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gla_scan: unknown dtype %d", dtype);
     FSIE_REQUIRE(proj && (z || head_decay) && state && q_starts && seq_slots && out && prep, "gla_scan: missing operand");
-    FSIE_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + heads * dim <= proj_stride &&
-                     k_off + heads * dim <= proj_stride && v_off + heads * vdim <= proj_stride,
+    FSIE_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && (qk || (q_off + heads * dim <= proj_stride &&
+                     k_off + heads * dim <= proj_stride)) && v_off + heads * vdim <= proj_stride,
                  "gla_scan: the q, k and v columns do not fit a row of %lld", static_cast<long long>(proj_stride));
     if (n_seqs == 0 || n_tokens == 0) return 0;
     int rows, splits;
@@ -320,7 +326,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
         FSIE_REQUIRE(max_chunks >= n_tokens / kGlaChunk + n_seqs, "gla_scan: room for %d chunks, the step may have %d",
                      max_chunks, n_tokens / kGlaChunk + n_seqs);
         FSIE_REQUIRE(max_chunks <= 0x7fffffff / kGlaChunk, "gla_scan: too many chunks");
-        FSIE_REQUIRE(proj_stride <= 0x7fffffff / kGlaChunk && static_cast<int64_t>(heads) * vdim <= 0x7fffffff / kGlaChunk,
+        FSIE_REQUIRE(proj_stride <= 0x7fffffff / kGlaChunk && qk_step <= 0x7fffffff / kGlaChunk && static_cast<int64_t>(heads) * vdim <= 0x7fffffff / kGlaChunk,
                      "gla_scan: rows too long for the chunk kernels' 32-bit offsets");
     }
     const int skip_from = chunks ? kGlaChunkMin : 0x7fffffff;
@@ -345,7 +351,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
                                                                state, q_starts, seq_slots, out, out_plane, heads, dim, vdim, \
                                                                dp, splits, n_slots, skip_from)
 #define FSIE_GLA_BY_ROWS(T)                                                                                          \
-    gla_prep_kernel<T><<<prep_grid, 256, 0, stream>>>(static_cast<const T*>(proj), proj_stride, q_off, k_off, z, prep, \
+    gla_prep_kernel<T><<<prep_grid, 256, 0, stream>>>(static_cast<const T*>(qk_rows), qk_step, q_off, k_off, z, prep, \
                                                       plane, heads, dim, dp, q_scale, inv_tau, q_starts, short_only, head_decay); \
     if (rows == 1) FSIE_GLA_LAUNCH(T, 1);                                                                            \
     else if (rows == 2) FSIE_GLA_LAUNCH(T, 2);                                                                       \
@@ -354,7 +360,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     else FSIE_GLA_LAUNCH(T, 16);                                                                                     \
     if (chunks) {                                                                                                    \
         gla_chunk_prep_kernel<T><<<chunk_grid, kGlaChunkThreads, chunk_lds, stream>>>(                                \
-            static_cast<const T*>(proj), proj_stride, q_off, k_off, z, chunk_work, q_starts, seq_slots, n_seqs, heads, dim, \
+            static_cast<const T*>(qk_rows), qk_step, q_off, k_off, z, chunk_work, q_starts, seq_slots, n_seqs, heads, dim, \
             dp, q_scale, inv_tau, n_slots, head_decay);                                                              \
         if (scan_waves == 1) FSIE_GLA_CHUNKS(T, 1);                                                                  \
         else if (scan_waves == 2) FSIE_GLA_CHUNKS(T, 2);                                                             \

@@ -858,7 +858,8 @@ def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
 # ---------------------------------------------------------------------------------------------
 def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, state: torch.Tensor,
              q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int, q_scale: float,
-             inv_tau: float, chunked: bool = True, head_decay: Optional[torch.Tensor] = None) -> torch.Tensor:
+             inv_tau: float, chunked: bool = True, head_decay: Optional[torch.Tensor] = None,
+             qk: Optional[torch.Tensor] = None) -> torch.Tensor:
     """S <- diag(sigmoid(z_t)^inv_tau) S + k_t v_t^T, o_t = S^T (q_scale q_t) over the tokens of every
     request of the step, from and to ``state`` float32 [slots, heads, dim, vdim].  ``proj`` [T, W] holds the
     q, k (heads x dim) and v (heads x vdim) columns from ``q_off``, ``k_off``, ``v_off``; ``z`` float32
@@ -882,6 +883,11 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
     n = seq_slots.shape[0]
     if q_starts.shape[0] != n + 1:
         raise KernelError("gla: q_starts must have one entry more than seq_slots")
+    if qk is not None:
+        # q and k in rows of their own [T, W'] (the same column offsets): what a caller has turned by the positions
+        _need(qk, "gla q and k", dtype=proj.dtype, ndim=2)
+        if qk.shape[0] != t:
+            raise KernelError("gla: a row of q and k a token")
     per_token, planes, chunk_tokens, chunk_min = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
     chunk_floats = ctypes.c_int64(0)
     check(load().fsie_gla_scan_shape(heads, dim, vdim, ctypes.byref(per_token), ctypes.byref(planes),
@@ -894,7 +900,8 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
     check(load().fsie_gla_scan(proj.data_ptr(), w, q_off, k_off, v_off, _ptr(z), state.data_ptr(), q_starts.data_ptr(),
                                seq_slots.data_ptr(), n, t, prep.data_ptr(), out.data_ptr(),
                                work.data_ptr() if work is not None else None, max_chunks, heads, dim, vdim, float(q_scale),
-                               float(inv_tau), state.shape[0], dtype_code(proj.dtype), _ptr(head_decay), _stream()))
+                               float(inv_tau), state.shape[0], dtype_code(proj.dtype), _ptr(head_decay), _ptr(qk),
+                               qk.shape[1] if qk is not None else 0, _stream()))
     return out
 
 

@@ -111,7 +111,7 @@ class AttentionPlanner:
 
     def uses_mfma(self, compute_dtype, page_size: int) -> bool:
         return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
-                and page_size % 4 == 0 and (not self.keep_first or self.mfma_keeps_first) and not self.pool)
+                and page_size % 4 == 0 and (not self.keep_first or self.mfma_keeps_first))
 
     mfma_keeps_first = True  # whether the matrix-core kernels read an item's kept first keys
 
@@ -271,7 +271,8 @@ class AttentionPlanner:
             if mine > 1:
                 longest = max(longest, split_keys)
                 mine += 1 if kept else 0  # (the kept first keys are an item of their own)
-                mine += 1 if self._pooled_seen(host.past_lens[s] + host.q_lens[s] - 1) else 0  # (and the pooled blocks)
+                if not mfma:  # (and the pooled blocks; the matrix-core geometry keeps them in a table of their own)
+                    mine += 1 if self._pooled_seen(host.past_lens[s] + host.q_lens[s] - 1) else 0
             elif kept:
                 longest = max(longest, keys + 32 * -(-kept // 32))
             n += mine
@@ -299,6 +300,17 @@ class AttentionPlanner:
         n_partial = 0
         pool_flag = ATTN_POOL_WALK if self.pool else 0
         pool_jobs = []
+        # The matrix-core kernels read keys and values of one pool.  With pooled blocks they leave partial records for
+        # the queries that see blocks, the float32-arithmetic kernel leaves the blocks' records (items of their own,
+        # ``pool_items``, cut to its tiles of queries), and the merge joins the two in one softmax.
+        two_pass = bool(mfma and self.pool)
+        pool_tile = ops.attention_tile_tokens(self.n_heads, self.n_kv) if two_pass else 0
+        pool_items, pooled_runs, merge_runs = [], [], []
+
+        def blocks_items(s, row0, n, p, base):
+            """The pooled blocks of n queries as items of the float32-arithmetic kernel, slots base .. base + n."""
+            for off in range(0, n, pool_tile):
+                pool_items.append((s, row0 + off, min(pool_tile, n - off), p + off, 0, 0, base + off, pool_flag))
         for s in range(host.n_seqs):
             if self.pool:
                 # the blocks whose last position this step brings: their means are made before attention runs
@@ -310,13 +322,16 @@ class AttentionPlanner:
                 keep = self.keep_first
                 total = p + n
                 n_splits = self._items_of(total - first_key, split_keys, most) if split_keys is not None else 1
-                if n <= small_tokens and n_splits > 1:
+                pooled = self._pooled_seen(total - 1) > 0
+                if n <= small_tokens and (n_splits > 1 or (two_pass and pooled)):
                     base = n_partial
                     if kept:
                         small.append((s, row0, n, p, 0, kept, base, keep))
                         base += n
-                    pooled = self._pooled_seen(total - 1) > 0
-                    if pooled:  # the pooled blocks: an item with no keys of its own
+                    if pooled and two_pass:
+                        blocks_items(s, row0, n, p, base)
+                        base += n
+                    elif pooled:  # the pooled blocks: an item with no keys of its own
                         small.append((s, row0, n, p, 0, 0, base, keep | pool_flag))
                         base += n
                     for i in range(n_splits):
@@ -327,7 +342,8 @@ class AttentionPlanner:
                         merges.append((row0 + t, n_partial + t, n_splits, n))
                     n_partial += n_splits * n
                 elif n <= small_tokens:
-                    small.append((s, row0, n, p, first_key, total, -1, (keep | ATTN_KEEP_WALK if keep else 0) | pool_flag))
+                    small.append((s, row0, n, p, first_key, total, -1,
+                                  (keep | ATTN_KEEP_WALK if keep else 0) | (0 if two_pass else pool_flag)))
                 else:
                     # (the short tile that a long portion may end with stays with the portion's other tiles:
                     # as a small item it would walk all the portion's keys in one workgroup a kv head, alone
@@ -344,8 +360,32 @@ class AttentionPlanner:
                         run[:, 4] = np.where(run[:, 4] <= self.keep_first, 0, run[:, 4])
                     run[:, 5] = pos0 + run[:, 2]
                     run[:, 6] = -1
-                    run[:, 7] = (self.keep_first | ATTN_KEEP_WALK if self.keep_first else 0) | pool_flag
-                    large_runs.append(run)
+                    run[:, 7] = (self.keep_first | ATTN_KEEP_WALK if self.keep_first else 0) | (0 if two_pass else pool_flag)
+                    if two_pass:
+                        # the tiles whose last query sees a block (the later ones of the run) leave partial records:
+                        # a tile of n_t queries has the slots base .. base + n_t for its keys, the next n_t for the blocks
+                        sees = np.maximum(0, run[:, 5] - self.window) // self.pool > 0
+                        mine, run = run[sees], run[~sees]
+                        if len(mine):
+                            n_t = mine[:, 2]
+                            ends = np.cumsum(2 * n_t)
+                            bases = n_partial + ends - 2 * n_t
+                            mine[:, 6] = bases
+                            tile = np.repeat(np.arange(len(mine)), n_t)
+                            t_in = np.arange(int(n_t.sum())) - np.repeat(np.cumsum(n_t) - n_t, n_t)
+                            merge_runs.append(np.stack([mine[tile, 1] + t_in, bases[tile] + t_in, np.full_like(t_in, 2), n_t[tile]], axis=1))
+                            pieces = -(-n_t // pool_tile)
+                            tile = np.repeat(np.arange(len(mine)), pieces)
+                            at = (np.arange(int(pieces.sum())) - np.repeat(np.cumsum(pieces) - pieces, pieces)) * pool_tile
+                            zeros = np.zeros_like(at)
+                            pooled_runs_items = np.stack([mine[tile, 0], mine[tile, 1] + at, np.minimum(pool_tile, n_t[tile] - at),
+                                                          mine[tile, 3] + at, zeros, zeros, bases[tile] + n_t[tile] + at,
+                                                          zeros + pool_flag], axis=1)
+                            pool_items += [tuple(int(v) for v in row) for row in pooled_runs_items]
+                            n_partial += int(ends[-1])
+                            pooled_runs.append(mine)
+                    if len(run):
+                        large_runs.append(run)
         large = np.concatenate(large_runs) if large_runs else np.zeros((0, ATTN_ITEM_INTS), dtype=np.int64)
         waves = 1
         if mfma and small:
@@ -358,12 +398,17 @@ class AttentionPlanner:
             if len(large) or len(small) > n_items:
                 raise RuntimeError("attention plan does not fit the captured graph")
             small += [(0, 0, 0, 0, 0, 0, -1, 0)] * (n_items - len(small))
-            if n_items > host.n_seqs:
+            if two_pass:
+                # one item of pooled blocks a request at most (a step of single tokens), and every row merged
+                if len(pool_items) > host.n_seqs:
+                    raise RuntimeError("attention plan: more items of pooled blocks than the captured graph has room for")
+                pool_items += [(0, 0, 0, 0, 0, 0, -1, 0)] * (host.n_seqs - len(pool_items))
+            if n_items > host.n_seqs or two_pass:
                 # the graph has room for items that share a request's keys: it merges every row
                 # (rows that need none get an empty merge)
                 merged = {m[0] for m in merges}
                 merges += [(row, 0, 0, 0) for row in range(host.n_tokens) if row not in merged]
-                n_partial = n_items * small_tokens
+                n_partial = (n_items + (host.n_seqs if two_pass else 0)) * small_tokens
         # consecutive large tiles of one request, four at a time, for the kernel that shares the
         # keys of a block among four waves
         groups = np.zeros((0, 2), dtype=np.int64)
@@ -380,8 +425,12 @@ class AttentionPlanner:
             # order of the requests would otherwise decide)
             order = np.argsort(large[firsts + counts - 1, 5] - large[firsts, 4], kind="stable")
             groups = np.stack([firsts[order], counts[order]], axis=1)
-        n_long = 0
-        if mfma and self.long_keys is not None:
+        n_long, long_waves = 0, 4
+        if pooled_runs:
+            # the tiles that leave partial records: a class of their own behind the others, a wave a workgroup
+            n_long, long_waves = sum(len(r) for r in pooled_runs), 1
+            large = np.concatenate([large] + pooled_runs)
+        elif mfma and self.long_keys is not None:
             # large tiles that read more than ``long_keys`` keys go to workgroups of four waves
             is_long = large[:, 5] - large[:, 4] > self.long_keys
             large = np.concatenate([large[~is_long], large[is_long]])
@@ -393,13 +442,15 @@ class AttentionPlanner:
                 if len(pool_jobs) > host.n_seqs:
                     raise RuntimeError("attention plan: more completed blocks than the captured graph has room for")
                 pool_jobs += [(-1, 0)] * (host.n_seqs - len(pool_jobs))
-            extra = {"pool_jobs": np.asarray(pool_jobs, dtype=np.int32).reshape(-1, 2), "n_pool_jobs": len(pool_jobs)}
+            extra = {"pool_jobs": np.asarray(pool_jobs, dtype=np.int32).reshape(-1, 2), "n_pool_jobs": len(pool_jobs),
+                     "pool_items": np.asarray(pool_items, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS), "n_pool_items": len(pool_items)}
         return {
             **extra,
             "items": np.concatenate([small_items, large]).astype(np.int32),
-            "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
+            "merges": np.concatenate([np.asarray(merges, dtype=np.int64).reshape(-1, ATTN_MERGE_INTS)] + merge_runs).astype(np.int32),
             "groups": groups.astype(np.int32), "n_groups": len(groups),
-            "n_small": len(small), "n_large": len(large) - n_long, "n_long": n_long, "n_merges": len(merges),
+            "n_small": len(small), "n_large": len(large) - n_long, "n_long": n_long, "long_waves": long_waves,
+            "n_merges": len(merges) + sum(len(m) for m in merge_runs),
             "n_partial": n_partial, "mfma": mfma, "waves": waves,
             "single": all(host.q_lens[s] == 1 for s in range(host.n_seqs)),  # one token a request
         }
@@ -417,8 +468,8 @@ def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n
     block_tokens): the pools of pooled blocks that items flagged ``ATTN_POOL_WALK`` read beside their keys (a planner
     with ``pool``).  Every mixer whose cache is pages of keys and values calls this."""
     cap = float(softcap or 0.0)
-    if pooled is not None and plan.mfma:
-        raise RuntimeError("attention: pooled blocks are read by the float32-arithmetic kernel alone")
+    if pooled is not None and plan.mfma and plan.n_pool_items and not plan.n_partial:
+        raise RuntimeError("attention: items of pooled blocks without partial records to leave them in")
     out = torch.empty((n_tokens, n_heads * head_dim), dtype=q.dtype, device=q.device)
     partials = None
     if plan.n_partial:
@@ -428,7 +479,8 @@ def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n
         if plan.n_small:
             ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
                                plan.n_small, out, *args, large=False, waves=plan.waves, sinks=sinks, softcap=cap)
-        if plan.n_large and not plan.n_long and share_keys and ops.attention_mfma_lds_ok(head_dim, cache.page_size):
+        if (plan.n_large and (not plan.n_long or getattr(plan, "long_waves", 4) == 1) and share_keys
+                and ops.attention_mfma_lds_ok(head_dim, cache.page_size)):
             ops.attention_mfma_lds(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
                                    plan.items[plan.n_small:], plan.groups, plan.n_groups, out, n_heads,
                                    n_kv, head_dim, window, scale, n_tokens, sinks=sinks, softcap=cap)
@@ -438,7 +490,11 @@ def paged_attention(q: torch.Tensor, q_stride: int, cache, plan, n_heads: int, n
         if plan.n_long:
             ops.attention_mfma(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables,
                                plan.items[plan.n_small + plan.n_large:], plan.n_long, out, *args, large=True,
-                               waves=4, sinks=sinks, softcap=cap)
+                               waves=getattr(plan, "long_waves", 4), sinks=sinks, softcap=cap)
+        if pooled is not None and plan.n_pool_items:
+            # the pooled blocks of the queries that see any: partial records beside those of their keys
+            ops.attention_scalar(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.pool_items,
+                                 plan.n_pool_items, out, *args, softcap=cap, pooled=pooled)
     else:
         ops.attention_scalar(q, q_stride, cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
                              plan.n_small + plan.n_large, out, *args, sinks=sinks, softcap=cap, pooled=pooled)

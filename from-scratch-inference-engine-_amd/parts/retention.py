@@ -75,13 +75,15 @@ class Retention(Mixer):
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         kw, vw = self.k_width, self.v_width
         p = self.qkvg(x)
+        turned = None
         if self.position.rotates:
+            # q and k turned into rows of their own (a lane reads its partner's value: not in place)
             pairs = self.position.rotary_dim // 2
-            turned = p[:, :2 * kw].contiguous()  # (a lane reads its partner's value: from a copy)
-            ops.rope_pairs(turned, 0, self.key_dim, p, 0, self.key_dim, 2 * self.n_heads, self.key_dim, -pairs, self.key_dim,
+            turned = torch.empty((p.shape[0], 2 * kw), dtype=p.dtype, device=p.device)
+            ops.rope_pairs(p, 0, self.key_dim, turned, 0, self.key_dim, 2 * self.n_heads, self.key_dim, -pairs, self.key_dim,
                            self.position.table(ctx))
         o = ops.gla_scan(p, 0, kw, 2 * kw, None, cache.state, ctx.q_starts, ctx.seq_slots, self.n_heads, self.key_dim,
-                         self.value_dim, self.key_scale, 1.0, head_decay=self._decay)
+                         self.value_dim, self.key_scale, 1.0, head_decay=self._decay, qk=turned)
         y = ops.gated_headnorm(o, p[:, 2 * kw + vw:], self._ones, self.norm_eps, self.n_heads, self.gate_activation)
         return self.o.for_residual(y, ctx)
 

@@ -94,7 +94,8 @@ def visible_by_definition(pos, window, chunk, pool):
 @pytest.mark.parametrize("window, chunk, pool", [(None, 16, None), (None, 1, None), (None, 7, None), (10, None, 4), (5, None, 7), (1, None, 1),
                                                  (96, None, 12), (None, None, None)])
 @pytest.mark.parametrize("units", [1, 256])
-def test_attention_plan_covers_what_a_query_reads(window, chunk, pool, units):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_plan_covers_what_a_query_reads(window, chunk, pool, units, dtype):
     """From the items alone, with the kernels' mask (causal, the window, the pooled blocks of flagged items): every query
     of a step reads exactly the keys and blocks of its definition, each once, and every block that the step completes is
     made."""
@@ -106,11 +107,24 @@ def test_attention_plan_covers_what_a_query_reads(window, chunk, pool, units):
         past = [int(rng.choice([0, 1, 15, 16, 17, 95, 96, 97, 300, 1500])) for _ in range(n_seqs)]
         new = [int(rng.choice([1, 1, 2, 3, 16, 33, 150])) for _ in range(n_seqs)]
         host = SimpleNamespace(n_seqs=n_seqs, q_lens=new, past_lens=past, q_starts=list(np.cumsum([0] + new)), page_size=16,
-                               compute_dtype=torch.float32, pad=None, memo={})
+                               compute_dtype=dtype, pad=None, memo={})
         host.n_tokens = host.q_starts[-1]
         plan = planner.plan(host)
         seen = {}  # row -> [keys list, blocks list]
-        for it in plan["items"]:
+        assert plan["mfma"] == (dtype == torch.bfloat16)
+        every = list(plan["items"]) + list(plan.get("pool_items", []))
+        assert not any(int(it[7]) & ATTN_POOL_WALK for it in plan["items"]) or not plan["mfma"]
+        slots = {}  # row -> slots of the partial records that items leave for it
+        for it in every:
+            if int(it[6]) >= 0:
+                for t in range(int(it[2])):
+                    slots.setdefault(int(it[1]) + t, []).append(int(it[6]) + t)
+        for row, first, n, stride in (tuple(int(v) for v in m) for m in plan["merges"]):
+            assert sorted(slots.pop(row)) == [first + i * stride for i in range(n)]
+        assert not slots and plan["n_merges"] == len(plan["merges"])
+        taken = [s for it in every if int(it[6]) >= 0 for s in range(int(it[6]), int(it[6]) + int(it[2]))]
+        assert len(taken) == len(set(taken)) and all(s < plan["n_partial"] for s in taken)
+        for it in every:
             s, row0, n, p, kb, ke, partial, flags = (int(v) for v in it)
             keep = flags & ~(ATTN_KEEP_WALK | ATTN_POOL_WALK)
             assert keep == 0
@@ -128,7 +142,7 @@ def test_attention_plan_covers_what_a_query_reads(window, chunk, pool, units):
                 keys, blocks = seen[row]
                 want_keys, want_blocks = visible_by_definition(pos, window, chunk, pool)
                 assert sorted(keys) == sorted(want_keys) and sorted(blocks) == sorted(want_blocks), (trial, s, t)
-        for it in plan["items"]:
+        for it in every:
             rows = range(int(it[1]), int(it[1]) + int(it[2]))
             assert all((r in merged) == (int(it[6]) >= 0) for r in rows)
         if pool:

@@ -201,7 +201,7 @@ def run_attention(case, heads, kv, hd, window, scale, cap=None, sinks=None, pool
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, kv, hd, page, chunk", [(4, 2, 64, 16, 64), (6, 1, 32, 8, 10), (2, 2, 48, 16, 7), (8, 2, 128, 16, 100),
-                                                        (3, 3, 20, 5, 1)])
+                                                        (3, 3, 20, 5, 1), (3, 1, 16, 8, 11), (6, 2, 16, 4, 5)])
 def test_chunked_attention_on_every_kernel(ops, dtype, heads, kv, hd, page, chunk):
     """A query reads the keys of its own chunk, counted from the request's start: decoded tokens at a chunk's first and
     last position, portions that start and end inside chunks and span several, first tokens.  Peaked rows: a key of
@@ -232,7 +232,8 @@ def test_chunked_attention_on_every_kernel(ops, dtype, heads, kv, hd, page, chun
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, kv, hd, page, window, pool, pooled_page", [(4, 2, 64, 16, 32, 8, 16), (6, 1, 32, 8, 10, 4, 8),
                                                                             (2, 2, 48, 16, 5, 7, 3), (3, 3, 20, 4, 1, 1, 4),
-                                                                            (4, 4, 64, 16, 96, 12, 16)])
+                                                                            (4, 4, 64, 16, 96, 12, 16), (6, 2, 32, 8, 9, 5, 8),
+                                                                            (3, 1, 16, 4, 7, 3, 2)])
 def test_window_with_pooled_blocks_a_sink_and_a_cap(ops, dtype, heads, kv, hd, page, window, pool, pooled_page):
     """The pooled blocks are made by the kernel from the cached keys and values (the mean of a block's positions), then
     every query reads its window, the blocks that lie wholly before it, and a sink of score 0: decoded tokens against long
@@ -252,7 +253,7 @@ def test_window_with_pooled_blocks_a_sink_and_a_cap(ops, dtype, heads, kv, hd, p
             case = attention_case(seqs, heads, kv, hd, page, dtype, seed=hd + pool, planner=planner, pool=pool, pooled_page=pooled_page)
         finally:
             AttentionPlanner.compute_units = None
-        assert not case["plan"]["mfma"]
+        assert case["plan"]["mfma"] == (dtype == torch.bfloat16 and hd % 16 == 0 and page % 4 == 0)
         # every whole block of every request, as if all its positions had come in this step
         jobs = [(s, b) for s, (p, n) in enumerate(seqs) for b in range((p + n) // pool)]
         pk, pv, ptab = case["pk"].cuda(), case["pv"].cuda(), case["ptab"].cuda()
@@ -514,7 +515,11 @@ CONFIG_D = {"architecture": "Mafosun", "width": 90, "vocab": 101, "norm": {"eps"
 CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
 
 
-def mafosun_tensors(cfg, seed):
+def mafosun_tensors(cfg, seed, sharp=True):
+    """``sharp``: head norms that make the softmax rows peaked and a router whose logits are far apart (the float32
+    tests: a key or an expert that is missed shows at once).  Not sharp: the same model with mild head norms and
+    router, for bfloat16, where a peaked row or a close choice turns a rounding of the input into another key or
+    another group of experts, which says nothing about the kernels."""
     g = torch.Generator().manual_seed(seed)
     w = cfg["width"]
 
@@ -528,7 +533,7 @@ def mafosun_tensors(cfg, seed):
     def attention_tensors(p, m):
         h, kv, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
         out.update({p + "q": mat(h * d, w), p + "k": mat(kv * d, w), p + "v": mat(kv * e, w), p + "o": mat(w, h * e),
-                    p + "q.norm": vec(d, 2.0, 0.3), p + "k.norm": vec(d, 2.0, 0.3)})  # (loud heads: peaked softmax rows)
+                    p + "q.norm": vec(d, 2.0 if sharp else 1.0, 0.3), p + "k.norm": vec(d, 2.0 if sharp else 1.0, 0.3)})
     for i, lay in enumerate(cfg["layers"]):
         m, p = lay["mixer"], f"l{i}.mix."
         out[f"l{i}.norm1"] = vec(w, 1.0, 0.2)
@@ -548,7 +553,7 @@ def mafosun_tensors(cfg, seed):
                 out.update({q + "gate": mat(mlp["ff"], w, 1.5), q + "up": mat(mlp["ff"], w, 1.5), q + "down": mat(w, mlp["ff"], 1.5)})
             else:
                 ff = mlp["expert"]["ff"]
-                out[q + "router"] = mat(mlp["router"]["experts"], w, 5.0)  # (spread logits: few choices are a rounding apart)
+                out[q + "router"] = mat(mlp["router"]["experts"], w, 10.0 if sharp else 4.0)
                 for j in range(mlp["router"]["experts"]):
                     out.update({f"{q}e{j}.gate": mat(ff, w, 1.5), f"{q}e{j}.up": mat(ff, w, 1.5), f"{q}e{j}.down": mat(w, ff, 1.5)})
     return {k: v.to(torch.bfloat16).contiguous() for k, v in out.items()}
@@ -559,16 +564,17 @@ def models(tmp_path_factory):
     root = tmp_path_factory.mktemp("mafosun")
     out = {}
     for name, cfg in CONFIGS.items():
-        d = helpers.make_model_dir(root / name, cfg, 0, tensors=mafosun_tensors(cfg, seed=ord(name)))
-        out[name] = (d, plain.read_config(d), plain.read_weights(d))
+        for tag, sharp in (("", True), ("~", False)):
+            d = helpers.make_model_dir(root / (name + tag), cfg, 0, tensors=mafosun_tensors(cfg, seed=ord(name), sharp=sharp))
+            out[name + tag] = (d, plain.read_config(d), plain.read_weights(d))
     return out
 
 
 def close_enough(got, ref, dtype, what):
     """float32: 1e-4 of the largest logit at every position.  bfloat16: the difference's root mean square against the
     logits'; with random weights the router's choice between two groups of experts is now and then a rounding apart,
-    and the other group is another function whose output the layer's norm brings to full size, so up to a fifth of the
-    positions may be far off while the typical one must be close."""
+    and the other group is another function whose output the layer's norm brings to full size, so a few positions may
+    be far off while the typical one must be close."""
     got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
     assert got.shape == ref.shape and np.isfinite(got).all(), what
     if dtype == "float32":
@@ -577,7 +583,7 @@ def close_enough(got, ref, dtype, what):
     else:
         err = np.sqrt(((got - ref) ** 2).mean(-1)) / np.sqrt((ref ** 2).mean())
         far = int((err > 0.12).sum())
-        assert far <= max(2, len(err) // 5) and np.median(err) <= 0.07, \
+        assert far <= max(1, len(err) // 10) and np.median(err) <= 0.06, \
             f"{what}: {far} of {len(err)} rows far off, the median row by {np.median(err):.3f} of the logits' size"
 
 
@@ -660,7 +666,7 @@ def test_model_whole_in_portions_decoded_and_batched(models, name, dtype):
     from from_scratch_inference_engine_amd import load_model
     from from_scratch_inference_engine_amd.engine.model import Runner
 
-    d, cfg, w = models[name]
+    d, cfg, w = models[name if dtype == "float32" else name + "~"]
     vocab = cfg["vocab"]
     seqs = {"a": helpers.token_ids(vocab, 75, 1), "b": helpers.token_ids(vocab, 1, 2), "c": helpers.token_ids(vocab, 33, 3),
             "d": helpers.token_ids(vocab, 130, 4), "e": helpers.token_ids(vocab, 18, 5)}
@@ -738,6 +744,7 @@ def test_replay_program_runs_the_model(models, tmp_path, name):
         tb.step(entries, end=["b"] if i == 19 else [])
     tb.step([("c", c, list(range(9)))], end=["a", "c"])
     for dtype in ("float32", "bfloat16"):
+        d, cfg, w = models[name if dtype == "float32" else name + "~"]
         per = helpers.collect(tb, helpers.run_trace(d, dtype, tb.steps, 128, tmp_path / dtype))
         for rid, ids in (("a", a), ("b", b), ("c", c)):
             ref = plain.forward(cfg, w, ids)
