@@ -84,7 +84,10 @@ int fsie_gla_scan_shape(int heads, int dim, int vdim, int* prep_floats_per_token
 int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, int k_off, int v_off, const float* z, float* state,
                   const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens, float* prep, float* out,
                   float* chunk_work, int max_chunks, int heads, int dim, int vdim, float q_scale, float inv_tau,
-                  int n_slots, int dtype, const float* head_decay, const void* qk, int64_t qk_stride, hipStream_t stream);
+                  int n_slots, int dtype, const float* head_decay, const void* qk, int64_t qk_stride, const float* cos_sin,
+                  int rot_pairs, hipStream_t stream);
+// cos_sin [n_tokens][rot_pairs][2] (or null and 0): the first 2 * rot_pairs channels of every q and k head are turned,
+// channel i with channel i + rot_pairs, by the token's cosines and sines as they are read (float32).
 // qk (or null): q and k are read from rows of their own, qk_stride values apart, at the same column offsets.
 // head_decay (or null): float32 [heads]; with it z may be null and every key channel of head h decays by head_decay[h],
 // the same for every token (retention: a fixed decay a head).

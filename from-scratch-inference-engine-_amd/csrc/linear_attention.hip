@@ -44,6 +44,18 @@ constexpr int kGlaChunkThreads = 256;
 // log(sigmoid(z)) without overflow: min(z, 0) - log(1 + exp(-|z|))
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
+// Channel i of a head's q or k (x points at it), turned by the token's angles where a rotation is given: the first
+// 2 * pairs channels of a head rotate, channel i with channel i + pairs, by cs[i mod pairs] = (cos, sin); float32.
+template <typename T>
+__device__ __forceinline__ float turned_channel(const T* __restrict__ x, int i, int pairs, const float2* __restrict__ cs) {
+    const float a = to_float(x[0]);
+    if (!cs || i >= 2 * pairs) return a;
+    const bool low = i < pairs;
+    const float b = to_float(low ? x[pairs] : x[-pairs]);
+    const float2 t = cs[low ? i : i - pairs];
+    return low ? fmaf(a, t.x, -(b * t.y)) : fmaf(a, t.x, b * t.y);
+}
+
 // prep [3][tokens][heads][dp]: scaled q, k, decay.  Grid: blocks of 256 elements over all tokens of the step,
 // or (with short_only > 0) over the first tokens of every request (grid.y), and only for requests of at most
 // short_only tokens: the others go chunk by chunk and need none of this.
@@ -51,7 +63,7 @@ template <typename T>
 __global__ void gla_prep_kernel(const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off,
                                 const float* __restrict__ z, float* __restrict__ prep, int64_t total, int heads, int dim,
                                 int dp, float q_scale, float inv_tau, const int32_t* __restrict__ q_starts, int short_only,
-                                const float* __restrict__ head_decay) {
+                                const float* __restrict__ head_decay, const float2* __restrict__ cos_sin, int pairs) {
     int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (short_only > 0) {
         const int lo = q_starts[blockIdx.y], len = q_starts[blockIdx.y + 1] - lo;
@@ -66,8 +78,9 @@ __global__ void gla_prep_kernel(const T* __restrict__ proj, int64_t proj_stride,
     float q = 0.f, k = 0.f, a = 1.f;
     if (i < dim) {
         const T* row = proj + t * proj_stride + h * dim + i;
-        q = to_float(row[q_off]) * q_scale;
-        k = to_float(row[k_off]);
+        const float2* cs = cos_sin ? cos_sin + t * pairs : nullptr;
+        q = turned_channel(row + q_off, i, pairs, cs) * q_scale;
+        k = turned_channel(row + k_off, i, pairs, cs);
         a = head_decay ? head_decay[h] : expf(inv_tau * log_sigmoid(z[(t * heads + h) * dim + i]));
     }
     prep[e] = q;
@@ -158,7 +171,8 @@ template <typename T>
 __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int q_off, int k_off, const float* __restrict__ z,
     float* __restrict__ work, const int32_t* __restrict__ q_starts, const int32_t* __restrict__ seq_slots, int n_seqs,
-    int heads, int dim, int dp, float q_scale, float inv_tau, int n_slots, const float* __restrict__ head_decay) {
+    int heads, int dim, int dp, float q_scale, float inv_tau, int n_slots, const float* __restrict__ head_decay,
+    const float2* __restrict__ cos_sin, int pairs) {
     extern __shared__ float lds[];  // [3][16][dp + 4]: q, k, B
     const int ld = dp + 4;
     float* qs = lds;
@@ -186,8 +200,9 @@ __global__ __launch_bounds__(kGlaChunkThreads) void gla_chunk_prep_kernel(
         float q = 0.f, k = 0.f, la = 0.f;
         if (t < nt && c < dim) {
             const T* row = proj + static_cast<int64_t>(t0 + t) * proj_stride + h * dim + c;
-            q = to_float(row[q_off]) * q_scale;
-            k = to_float(row[k_off]);
+            const float2* cs = cos_sin ? cos_sin + static_cast<int64_t>(t0 + t) * pairs : nullptr;
+            q = turned_channel(row + q_off, c, pairs, cs) * q_scale;
+            k = turned_channel(row + k_off, c, pairs, cs);
             la = head_decay ? log2f(head_decay[h])
                             : to_log2 * log_sigmoid(z[(static_cast<int64_t>(t0 + t) * heads + h) * dim + c]);
         }
@@ -298,7 +313,10 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
                              float* state, const int32_t* q_starts, const int32_t* seq_slots, int n_seqs, int n_tokens,
                              float* prep, float* out, float* chunk_work, int max_chunks, int heads, int dim, int vdim,
                              float q_scale, float inv_tau, int n_slots, int dtype, const float* head_decay,
-                             const void* qk, int64_t qk_stride, hipStream_t stream) {
+                             const void* qk, int64_t qk_stride, const float* cos_sin, int rot_pairs, hipStream_t stream) {
+    FSIE_REQUIRE(rot_pairs >= 0 && 2 * rot_pairs <= dim && (rot_pairs == 0 || cos_sin), "gla_scan: %d rotated pairs in heads of %d",
+                 rot_pairs, dim);
+    const float2* turn = rot_pairs > 0 ? reinterpret_cast<const float2*>(cos_sin) : nullptr;
     // q and k may live in rows of their own (qk, rows qk_stride apart, the same column offsets): a caller that has
     // turned them by the positions without touching the projection
     const void* qk_rows = qk ? qk : proj;
@@ -352,7 +370,8 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
                                                                dp, splits, n_slots, skip_from)
 #define FSIE_GLA_BY_ROWS(T)                                                                                          \
     gla_prep_kernel<T><<<prep_grid, 256, 0, stream>>>(static_cast<const T*>(qk_rows), qk_step, q_off, k_off, z, prep, \
-                                                      plane, heads, dim, dp, q_scale, inv_tau, q_starts, short_only, head_decay); \
+                                                      plane, heads, dim, dp, q_scale, inv_tau, q_starts, short_only, head_decay,  \
+                                                      turn, rot_pairs);                                              \
     if (rows == 1) FSIE_GLA_LAUNCH(T, 1);                                                                            \
     else if (rows == 2) FSIE_GLA_LAUNCH(T, 2);                                                                       \
     else if (rows == 4) FSIE_GLA_LAUNCH(T, 4);                                                                       \
@@ -361,7 +380,7 @@ extern "C" int fsie_gla_scan(const void* proj, int64_t proj_stride, int q_off, i
     if (chunks) {                                                                                                    \
         gla_chunk_prep_kernel<T><<<chunk_grid, kGlaChunkThreads, chunk_lds, stream>>>(                                \
             static_cast<const T*>(qk_rows), qk_step, q_off, k_off, z, chunk_work, q_starts, seq_slots, n_seqs, heads, dim, \
-            dp, q_scale, inv_tau, n_slots, head_decay);                                                              \
+            dp, q_scale, inv_tau, n_slots, head_decay, turn, rot_pairs);                                             \
         if (scan_waves == 1) FSIE_GLA_CHUNKS(T, 1);                                                                  \
         else if (scan_waves == 2) FSIE_GLA_CHUNKS(T, 2);                                                             \
         else if (scan_waves == 4) FSIE_GLA_CHUNKS(T, 4);                                                             \

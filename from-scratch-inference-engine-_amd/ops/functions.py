@@ -859,7 +859,7 @@ def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
 def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, state: torch.Tensor,
              q_starts: torch.Tensor, seq_slots: torch.Tensor, heads: int, dim: int, vdim: int, q_scale: float,
              inv_tau: float, chunked: bool = True, head_decay: Optional[torch.Tensor] = None,
-             qk: Optional[torch.Tensor] = None) -> torch.Tensor:
+             qk: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
     """S <- diag(sigmoid(z_t)^inv_tau) S + k_t v_t^T, o_t = S^T (q_scale q_t) over the tokens of every
     request of the step, from and to ``state`` float32 [slots, heads, dim, vdim].  ``proj`` [T, W] holds the
     q, k (heads x dim) and v (heads x vdim) columns from ``q_off``, ``k_off``, ``v_off``; ``z`` float32
@@ -888,6 +888,14 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
         _need(qk, "gla q and k", dtype=proj.dtype, ndim=2)
         if qk.shape[0] != t:
             raise KernelError("gla: a row of q and k a token")
+    rot_pairs = 0
+    if cos_sin is not None:
+        # the step's cosines and sines [T, pairs, 2]: the first 2 * pairs channels of every q and k head are turned as
+        # they are read, channel i with channel i + pairs
+        _need(cos_sin, "gla cos/sin", dtype=torch.float32, ndim=3)
+        rot_pairs = cos_sin.shape[1]
+        if tuple(cos_sin.shape) != (t, rot_pairs, 2) or 2 * rot_pairs > dim:
+            raise KernelError(f"gla: cosines and sines {tuple(cos_sin.shape)} do not fit {t} tokens and heads of {dim}")
     per_token, planes, chunk_tokens, chunk_min = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
     chunk_floats = ctypes.c_int64(0)
     check(load().fsie_gla_scan_shape(heads, dim, vdim, ctypes.byref(per_token), ctypes.byref(planes),
@@ -901,7 +909,7 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
                                seq_slots.data_ptr(), n, t, prep.data_ptr(), out.data_ptr(),
                                work.data_ptr() if work is not None else None, max_chunks, heads, dim, vdim, float(q_scale),
                                float(inv_tau), state.shape[0], dtype_code(proj.dtype), _ptr(head_decay), _ptr(qk),
-                               qk.shape[1] if qk is not None else 0, _stream()))
+                               qk.shape[1] if qk is not None else 0, _ptr(cos_sin), rot_pairs, _stream()))
     return out
 
 

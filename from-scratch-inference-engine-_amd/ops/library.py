@@ -81,7 +81,7 @@ _SIGNATURES = {
                              ctypes.POINTER(c_int), ctypes.POINTER(c_int64)], c_int),
     "fsie_softcap": ([_P, c_int64, c_float, _P], c_int),
     "fsie_gla_scan": ([_P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int, _P, _P, _P, c_int, c_int, c_int, c_int,
-                       c_float, c_float, c_int, c_int, _P, _P, c_int64, _P], c_int),
+                       c_float, c_float, c_int, c_int, _P, _P, c_int64, _P, c_int, _P], c_int),
     "fsie_latent_prep": ([_P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, _P, _P,
                           _P, _P, _P, c_int, c_int, c_int64, c_int, c_int, _P], c_int),
     "fsie_rope_pairs": ([_P, c_int64, c_int, c_int, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P, c_int, c_int,

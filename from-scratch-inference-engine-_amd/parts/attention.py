@@ -305,7 +305,7 @@ class AttentionPlanner:
         # ``pool_items``, cut to its tiles of queries), and the merge joins the two in one softmax.
         two_pass = bool(mfma and self.pool)
         pool_tile = ops.attention_tile_tokens(self.n_heads, self.n_kv) if two_pass else 0
-        pool_items, pooled_runs, merge_runs = [], [], []
+        pool_items, pool_item_runs, pooled_runs, merge_runs = [], [], [], []
 
         def blocks_items(s, row0, n, p, base):
             """The pooled blocks of n queries as items of the float32-arithmetic kernel, slots base .. base + n."""
@@ -378,10 +378,9 @@ class AttentionPlanner:
                             tile = np.repeat(np.arange(len(mine)), pieces)
                             at = (np.arange(int(pieces.sum())) - np.repeat(np.cumsum(pieces) - pieces, pieces)) * pool_tile
                             zeros = np.zeros_like(at)
-                            pooled_runs_items = np.stack([mine[tile, 0], mine[tile, 1] + at, np.minimum(pool_tile, n_t[tile] - at),
-                                                          mine[tile, 3] + at, zeros, zeros, bases[tile] + n_t[tile] + at,
-                                                          zeros + pool_flag], axis=1)
-                            pool_items += [tuple(int(v) for v in row) for row in pooled_runs_items]
+                            pool_item_runs.append(np.stack([mine[tile, 0], mine[tile, 1] + at, np.minimum(pool_tile, n_t[tile] - at),
+                                                            mine[tile, 3] + at, zeros, zeros, bases[tile] + n_t[tile] + at,
+                                                            zeros + pool_flag], axis=1))
                             n_partial += int(ends[-1])
                             pooled_runs.append(mine)
                     if len(run):
@@ -443,7 +442,9 @@ class AttentionPlanner:
                     raise RuntimeError("attention plan: more completed blocks than the captured graph has room for")
                 pool_jobs += [(-1, 0)] * (host.n_seqs - len(pool_jobs))
             extra = {"pool_jobs": np.asarray(pool_jobs, dtype=np.int32).reshape(-1, 2), "n_pool_jobs": len(pool_jobs),
-                     "pool_items": np.asarray(pool_items, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS), "n_pool_items": len(pool_items)}
+                     "pool_items": np.concatenate([np.asarray(pool_items, dtype=np.int64).reshape(-1, ATTN_ITEM_INTS)]
+                                                  + pool_item_runs).astype(np.int32),
+                     "n_pool_items": len(pool_items) + sum(len(r) for r in pool_item_runs)}
         return {
             **extra,
             "items": np.concatenate([small_items, large]).astype(np.int32),

@@ -25,7 +25,7 @@ class Retention(Mixer):
     projected by W_o.  The projections that read x are one matrix (q, k, v, g rows one after the other).
 
     The state lives in the cache manager's per-request slots, zero when a request starts; decays, state and sums
-    are float32 whatever the activations' type.  The walk over a request's tokens is the one of gated linear
+    are float32 whatever the activations' type.  The rotation happens in float32 inside the scan's first kernel.  The walk over a request's tokens is the one of gated linear
     attention (token by token, or chunk by chunk on the float32 matrix instruction for long portions) with the
     head's decay in the place of a decay per token and key channel."""
 
@@ -75,15 +75,10 @@ class Retention(Mixer):
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         kw, vw = self.k_width, self.v_width
         p = self.qkvg(x)
-        turned = None
-        if self.position.rotates:
-            # q and k turned into rows of their own (a lane reads its partner's value: not in place)
-            pairs = self.position.rotary_dim // 2
-            turned = torch.empty((p.shape[0], 2 * kw), dtype=p.dtype, device=p.device)
-            ops.rope_pairs(p, 0, self.key_dim, turned, 0, self.key_dim, 2 * self.n_heads, self.key_dim, -pairs, self.key_dim,
-                           self.position.table(ctx))
+        # (the scan's own first kernel turns q and k by the step's cosines and sines as it reads them)
+        table = self.position.table(ctx) if self.position.rotates else None
         o = ops.gla_scan(p, 0, kw, 2 * kw, None, cache.state, ctx.q_starts, ctx.seq_slots, self.n_heads, self.key_dim,
-                         self.value_dim, self.key_scale, 1.0, head_decay=self._decay, qk=turned)
+                         self.value_dim, self.key_scale, 1.0, head_decay=self._decay, cos_sin=table)
         y = ops.gated_headnorm(o, p[:, 2 * kw + vw:], self._ones, self.norm_eps, self.n_heads, self.gate_activation)
         return self.o.for_residual(y, ctx)
 

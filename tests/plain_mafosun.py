@@ -158,9 +158,12 @@ def retention(q, k, v, decay):
     return out
 
 
-def route(z, top, groups, keep):
+def route(z, top, groups, keep, margins=None):
     """Softmax scores over all experts; only experts of the ``keep`` groups with the largest best score can be
-    chosen; the ``top`` largest scores among them, and those scores as weights.  Returns (ids [T, top], weights)."""
+    chosen; the ``top`` largest scores among them, and those scores as weights.  Returns (ids [T, top], weights).
+    ``margins`` (a list) receives, per token, by how much of the logits' spread the choice was made: the smaller of the
+    distance between the last group kept and the first one dropped and between the last expert chosen and the first
+    one not (infinite where there is nothing to drop)."""
     s = np.exp(z - z.max(-1, keepdims=True))
     s /= s.sum(-1, keepdims=True)
     t, experts = s.shape
@@ -174,6 +177,12 @@ def route(z, top, groups, keep):
             allowed[g * per:(g + 1) * per] = s[i, g * per:(g + 1) * per]
         chosen = np.argsort(-allowed, kind="stable")[:top]
         ids[i], weights[i] = chosen, s[i, chosen]
+        if margins is not None:
+            by_group = np.sort(z[i].reshape(groups, per).max(1))[::-1]
+            inside = np.sort(np.where(np.isfinite(allowed), z[i], -np.inf))[::-1]
+            gap = min(by_group[keep - 1] - by_group[keep] if keep < groups else np.inf,
+                      inside[top - 1] - inside[top] if top < keep * per else np.inf)
+            margins.append(gap / max(z[i].max() - z[i].min(), 1e-30))
     return ids, weights
 
 
@@ -229,9 +238,9 @@ def dense_ff(h, w, p):
     return (np.maximum(h @ w[p + "gate"].T, 0.0) * (h @ w[p + "up"].T)) @ w[p + "down"].T
 
 
-def expert_ff(h, w, p, mlp):
+def expert_ff(h, w, p, mlp, margins=None):
     r = mlp["router"]
-    ids, weights = route(h @ w[p + "router"].T, r["top"], r["groups"]["count"], r["groups"]["keep"])
+    ids, weights = route(h @ w[p + "router"].T, r["top"], r["groups"]["count"], r["groups"]["keep"], margins)
     out = np.zeros_like(h)
     for i in range(h.shape[0]):
         for e, a in zip(ids[i], weights[i]):
@@ -240,8 +249,9 @@ def expert_ff(h, w, p, mlp):
     return out
 
 
-def forward(cfg: dict, w: dict, tokens, streams=None):
-    """Logits [T, vocab] of the whole sequence ``tokens``; ``streams`` (a list) receives the stream after each layer."""
+def forward(cfg: dict, w: dict, tokens, streams=None, margins=None):
+    """Logits [T, vocab] of the whole sequence ``tokens``; ``streams`` (a list) receives the stream after each layer,
+    ``margins`` (a list) one array [T] for every layer of routed experts: how clear each token's choice was."""
     eps = cfg["norm"]["eps"]
     tokens = np.asarray(tokens, dtype=np.int64)
     positions = np.arange(tokens.shape[0])
@@ -257,7 +267,13 @@ def forward(cfg: dict, w: dict, tokens, streams=None):
         x = x + rms_norm(y, w[p + "norm1"], eps)
         mlp = layer.get("mlp")
         if mlp is not None:
-            y = dense_ff(x, w, p + "mlp.") if mlp["kind"] == "dense" else expert_ff(x, w, p + "mlp.", mlp)
+            if mlp["kind"] == "dense":
+                y = dense_ff(x, w, p + "mlp.")
+            else:
+                mine = [] if margins is not None else None
+                y = expert_ff(x, w, p + "mlp.", mlp, mine)
+                if margins is not None:
+                    margins.append(np.asarray(mine))
             x = x + rms_norm(y, w[p + "norm2"], eps)
         if streams is not None:
             streams.append(x.copy())

@@ -369,16 +369,21 @@ def test_retention_over_portions_steps_and_slots(ops, dtype, heads, dim, vdim, d
     fed, got = {r: 0 for r in lens}, {r: [] for r in lens}
     decay = torch.tensor(decays, dtype=torch.float32).cuda()
     scale = dim ** -0.5
+    rot = dim // 4 * 2  # the first channels of every q and k head turn by the position, inside the scan's first kernel
+    freqs = plain.rotary_frequencies(rot, 300.0)
     for step in plan:
-        rows, starts, slots = [], [0], []
+        rows, starts, slots, pos = [], [0], [], []
         for r, n in step:
             if fed[r] == 0:
                 state[slot[r]] = 0.0  # (the engine zeroes the slots of the requests that start)
             rows.append(proj[r][fed[r]:fed[r] + n])
+            pos += list(range(fed[r], fed[r] + n))
             starts.append(starts[-1] + n)
             slots.append(slot[r])
+        ang = np.asarray(pos, dtype=np.float64)[:, None] * freqs[None, :]
+        table = torch.tensor(np.stack([np.cos(ang), np.sin(ang)], -1), dtype=torch.float32).cuda()
         o = ops.gla_scan(torch.cat(rows).cuda(), 0, heads * dim, 2 * heads * dim, None, state, i32(starts), i32(slots), heads, dim,
-                         vdim, scale, 1.0, head_decay=decay).sum(0).cpu()
+                         vdim, scale, 1.0, head_decay=decay, cos_sin=table).sum(0).cpu()
         at = 0
         for r, n in step:
             got[r].append(o[at:at + n])
@@ -386,7 +391,8 @@ def test_retention_over_portions_steps_and_slots(ops, dtype, heads, dim, vdim, d
             fed[r] += n
     for r, n in lens.items():
         p = proj[r].double().numpy()
-        q, k = p[:, :heads * dim].reshape(n, heads, dim), p[:, heads * dim:2 * heads * dim].reshape(n, heads, dim) * scale
+        q, k = p[:, :heads * dim].reshape(n, heads, dim), p[:, heads * dim:2 * heads * dim].reshape(n, heads, dim)
+        q, k = plain.rotate(q, np.arange(n), freqs, rot, "half"), plain.rotate(k, np.arange(n), freqs, rot, "half") * scale
         ref = plain.retention(q, k, p[:, 2 * heads * dim:].reshape(n, heads, vdim), decays).reshape(n, heads * vdim)
         assert rel(torch.cat(got[r]), ref) <= 2e-5, r  # (the scan is float32 whatever the inputs' type)
 
@@ -516,10 +522,9 @@ CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
 
 
 def mafosun_tensors(cfg, seed, sharp=True):
-    """``sharp``: head norms that make the softmax rows peaked and a router whose logits are far apart (the float32
-    tests: a key or an expert that is missed shows at once).  Not sharp: the same model with mild head norms and
-    router, for bfloat16, where a peaked row or a close choice turns a rounding of the input into another key or
-    another group of experts, which says nothing about the kernels."""
+    """``sharp``: head norms that make the softmax rows peaked (the float32 tests: a key that is missed shows at once).
+    Not sharp: the same tensors with mild head norms, for bfloat16, where a peaked row turns a rounding of the input
+    into another key, which says nothing about the kernels (those models also use all their experts: ``without_choices``)."""
     g = torch.Generator().manual_seed(seed)
     w = cfg["width"]
 
@@ -553,10 +558,23 @@ def mafosun_tensors(cfg, seed, sharp=True):
                 out.update({q + "gate": mat(mlp["ff"], w, 1.5), q + "up": mat(mlp["ff"], w, 1.5), q + "down": mat(w, mlp["ff"], 1.5)})
             else:
                 ff = mlp["expert"]["ff"]
-                out[q + "router"] = mat(mlp["router"]["experts"], w, 10.0 if sharp else 4.0)
+                out[q + "router"] = mat(mlp["router"]["experts"], w, 10.0)  # (logits far apart: few choices are a rounding apart)
                 for j in range(mlp["router"]["experts"]):
                     out.update({f"{q}e{j}.gate": mat(ff, w, 1.5), f"{q}e{j}.up": mat(ff, w, 1.5), f"{q}e{j}.down": mat(w, ff, 1.5)})
     return {k: v.to(torch.bfloat16).contiguous() for k, v in out.items()}
+
+
+def without_choices(cfg):
+    """The same configuration with every expert chosen (all groups kept, top = experts): the weights are the softmax
+    scores, a continuous function of the input.  For whole models in bfloat16, where a choice between two groups of
+    experts that is made by a hair falls either way and the other group is another function; the choice itself is
+    tested alone in both types and in whole models in float32."""
+    cfg = copy.deepcopy(cfg)
+    for lay in cfg["layers"]:
+        if lay["mlp"] is not None and lay["mlp"]["kind"] == "moe":
+            r = lay["mlp"]["router"]
+            r["top"], r["groups"]["keep"] = r["experts"], r["groups"]["count"]
+    return cfg
 
 
 @pytest.fixture(scope="module")
@@ -565,9 +583,22 @@ def models(tmp_path_factory):
     out = {}
     for name, cfg in CONFIGS.items():
         for tag, sharp in (("", True), ("~", False)):
-            d = helpers.make_model_dir(root / (name + tag), cfg, 0, tensors=mafosun_tensors(cfg, seed=ord(name), sharp=sharp))
+            d = helpers.make_model_dir(root / (name + tag), cfg if sharp else without_choices(cfg), 0,
+                                       tensors=mafosun_tensors(cfg, seed=ord(name), sharp=sharp))
             out[name + tag] = (d, plain.read_config(d), plain.read_weights(d))
     return out
+
+
+def clear_rows(cfg, w, ids, least=0.03):
+    """The first positions of a sequence up to the first token whose choice of experts, in any layer, is made by less
+    than ``least`` of its logits' spread.  In bfloat16 such a choice can fall the other way; the other group of experts
+    is another function, and what it writes reaches every later position through keys, values and states."""
+    margins = []
+    plain.forward(cfg, w, ids, margins=margins)
+    if not margins:
+        return len(ids)
+    close = np.nonzero(np.min(np.stack(margins), axis=0) < least)[0]
+    return int(close[0]) if len(close) else len(ids)
 
 
 def close_enough(got, ref, dtype, what):
@@ -671,27 +702,34 @@ def test_model_whole_in_portions_decoded_and_batched(models, name, dtype):
     seqs = {"a": helpers.token_ids(vocab, 75, 1), "b": helpers.token_ids(vocab, 1, 2), "c": helpers.token_ids(vocab, 33, 3),
             "d": helpers.token_ids(vocab, 130, 4), "e": helpers.token_ids(vocab, 18, 5)}
     ref = {r: plain.forward(cfg, w, ids) for r, ids in seqs.items()}
+    # bfloat16: a request is compared up to its first token whose choice of experts is a close call
+    upto = {r: len(ids) if dtype == "float32" else clear_rows(cfg, w, ids) for r, ids in seqs.items()}
+    assert dtype == "float32" or sum(upto.values()) >= sum(len(ids) for ids in seqs.values()) // 3
     model = load_model(d, dtype=dtype)
     runner = Runner(model, page_size=8, num_pages=40, max_requests=3)
     assert runner.graphs.enabled
+
+    def check(got, r, what):
+        if upto[r]:
+            close_enough(got[r][:upto[r]], ref[r][:upto[r]], dtype, what)
     got = step_through(runner, [[(r, len(ids))] for r, ids in seqs.items()], seqs)
     for r in seqs:
-        close_enough(got[r], ref[r], dtype, f"{name} whole {r}")
+        check(got, r, f"{name} whole {r}")
     for r, head in (("a", 10), ("c", 1)):
         got = step_through(runner, [[(r, head)]] + [[(r, 1)]] * (len(seqs[r]) - head), {r: seqs[r]})
-        close_enough(got[r], ref[r], dtype, f"{name} decode {r}")
+        check(got, r, f"{name} decode {r}")
     assert runner.graphs.replays > 50
     sizes, plan, left = [2, 7, 1, 16, 3, 2, 33, 8, 64], [], len(seqs["d"])
     while left:
         n = min(sizes[len(plan) % len(sizes)], left)
         plan.append([("d", n)])
         left -= n
-    close_enough(step_through(runner, plan, {"d": seqs["d"]})["d"], ref["d"], dtype, f"{name} portions")
+    check(step_through(runner, plan, {"d": seqs["d"]}), "d", f"{name} portions")
     plan = [[("a", 30), ("c", 2), ("b", 1)], [("a", 1), ("c", 20), ("e", 3)], [("c", 11), ("a", 44), ("e", 1)],
             [("e", 14), ("d", 9)], [("d", 120)], [("d", 1)]]
     got = step_through(runner, plan, seqs)
     for r in seqs:
-        close_enough(got[r], ref[r], dtype, f"{name} batched {r}")
+        check(got, r, f"{name} batched {r}")
     assert all(a.pages_issued_again() for a in runner.manager.allocators)
 
 
@@ -748,8 +786,10 @@ def test_replay_program_runs_the_model(models, tmp_path, name):
         per = helpers.collect(tb, helpers.run_trace(d, dtype, tb.steps, 128, tmp_path / dtype))
         for rid, ids in (("a", a), ("b", b), ("c", c)):
             ref = plain.forward(cfg, w, ids)
-            pos = sorted(per[rid])
-            close_enough(np.stack([per[rid][p] for p in pos]), ref[pos], dtype, f"replay {rid}")
+            upto = len(ids) if dtype == "float32" else clear_rows(cfg, w, ids)
+            pos = [p for p in sorted(per[rid]) if p < upto]
+            if pos:
+                close_enough(np.stack([per[rid][p] for p in pos]), ref[pos], dtype, f"replay {rid}")
 
 
 def test_command_line_writes_a_random_model_and_generates(tmp_path):
