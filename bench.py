@@ -285,8 +285,8 @@ def fiterax_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
 
 
 def mafosun_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
-    """A Mafosun configuration of real layer sizes: layers of chunked attention beside retention and layers of attention
-    over a window of 1,024 positions with pooled blocks of 64 in turn, a dense feed-forward and eight routed experts in
+    """A Mafosun configuration of real layer sizes: layers of chunked attention (chunks of 1,024 positions) beside
+    retention and layers of attention over a window of 1,024 positions with pooled blocks of 64 in turn, a dense feed-forward and eight routed experts in
     two groups (two a token, from the best group) in turn; an expert has gate, up and down of ff / 8, so a token's two
     experts are a quarter of the dense feed-forward's arithmetic."""
     heads = width // 128
@@ -294,7 +294,7 @@ def mafosun_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
     gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
            "mask": {"size": 1024, "pool": 64}, "rot": {"base": 500000.0, "dims": 64, "scaling": bands}}
     pair = {"left": {"heads": heads // 2, "kv_heads": max(1, width // 1024), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                     "mask": {"size": 512}},
+                     "mask": {"size": 1024}},
             "right": {"heads": width // 256, "dim": 128, "vdim": 128, "rot": {"base": 500000.0, "dims": 128},
                       "decay": [1.0 - 2.0 ** -(5 + i % 6) for i in range(width // 256)]},
             "left_scale": 1.2, "right_scale": 0.5}

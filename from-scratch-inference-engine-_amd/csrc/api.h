@@ -213,7 +213,8 @@ int fsie_attention_merge(const float* partials, const int32_t* merges, int n_mer
 int fsie_attention_scalar_tile_tokens(int n_heads, int n_kv);
 // The mean key and value of blocks of `block_tokens` consecutive positions, from the pages of keys and values to the
 // pools of pooled blocks: jobs [n_jobs][2] = (request of the step, block), a request of -1: nothing.  Block b's
-// positions b * block_tokens .. are read through the request's row of block_tables and summed in their order in float32;
+// positions b * block_tokens .. are read through the request's row of block_tables and summed in float32 in a fixed order
+// (runs of consecutive positions, each in its order, then the runs in theirs);
 // the entry goes to the page that pooled_tables names for b.
 int fsie_pool_blocks(const void* k_pool, const void* v_pool, const int32_t* block_tables, int max_pages, int page_size,
                      void* k_pooled, void* v_pooled, const int32_t* pooled_tables, int pooled_max_pages, int pooled_page_size,

@@ -396,14 +396,16 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     }
 }
 
-// One workgroup a job and kv head, a thread a dimension (in turns): the sums run over the block's positions in order.
+// One workgroup a job and kv head: 256 threads as `parts` runs of positions by a dimension each (parts = 256 / head
+// size rounded up to a power of two, at least one); a run's positions are added in their order, the runs in theirs.
 template <typename T>
 __global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ k_pool, const T* __restrict__ v_pool,
                                                           const int32_t* __restrict__ block_tables, int max_pages,
                                                           int page_size, T* __restrict__ k_pooled, T* __restrict__ v_pooled,
                                                           const int32_t* __restrict__ pooled_tables, int pooled_max_pages,
                                                           int pooled_page_size, const int32_t* __restrict__ jobs,
-                                                          int block_tokens, int n_kv, int hd) {
+                                                          int block_tokens, int n_kv, int hd, int lanes) {
+    __shared__ float s_sum[2][256];
     const int seq = jobs[2 * blockIdx.x], block = jobs[2 * blockIdx.x + 1];
     if (seq < 0) return;
     const int kvh = blockIdx.y;
@@ -412,18 +414,30 @@ __global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ 
     if (to_page < 0) return;
     const int to_off = block % pooled_page_size;
     const float inv = 1.0f / static_cast<float>(block_tokens);
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    const int parts = 256 / lanes, part = threadIdx.x / lanes, lane = threadIdx.x % lanes;
+    const int per = (block_tokens + parts - 1) / parts;  // positions a run
+    for (int d0 = 0; d0 < hd; d0 += lanes) {
+        const int d = d0 + lane;
         float ks = 0.f, vs = 0.f;
-        for (int i = 0; i < block_tokens; ++i) {
-            const int pos = block * block_tokens + i;
-            const int page = table[pos / page_size];
-            if (page < 0) continue;
-            const int off = pos % page_size;
-            ks += to_float(k_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + off) * hd + d]);
-            vs += to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + off]);
+        if (d < hd) {
+            for (int i = part * per; i < min(block_tokens, (part + 1) * per); ++i) {
+                const int pos = block * block_tokens + i;
+                const int page = table[pos / page_size];
+                if (page < 0) continue;
+                const int off = pos % page_size;
+                ks += to_float(k_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + off) * hd + d]);
+                vs += to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + off]);
+            }
         }
-        k_pooled[((static_cast<int64_t>(to_page) * n_kv + kvh) * pooled_page_size + to_off) * hd + d] = from_float<T>(ks * inv);
-        v_pooled[((static_cast<int64_t>(to_page) * n_kv + kvh) * hd + d) * pooled_page_size + to_off] = from_float<T>(vs * inv);
+        __syncthreads();  // (the sums of the dimensions before have been read)
+        s_sum[0][threadIdx.x] = ks;
+        s_sum[1][threadIdx.x] = vs;
+        __syncthreads();
+        if (part == 0 && d < hd) {
+            for (int p = 1; p < parts; ++p) ks += s_sum[0][p * lanes + lane], vs += s_sum[1][p * lanes + lane];
+            k_pooled[((static_cast<int64_t>(to_page) * n_kv + kvh) * pooled_page_size + to_off) * hd + d] = from_float<T>(ks * inv);
+            v_pooled[((static_cast<int64_t>(to_page) * n_kv + kvh) * hd + d) * pooled_page_size + to_off] = from_float<T>(vs * inv);
+        }
     }
 }
 
@@ -511,17 +525,19 @@ extern "C" int fsie_pool_blocks(const void* k_pool, const void* v_pool, const in
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "pool_blocks: unknown dtype %d", dtype);
     if (n_jobs == 0) return 0;
     const dim3 grid(n_jobs, n_kv);
-    const int threads = head_dim <= 64 ? 64 : (head_dim <= 128 ? 128 : 256);
+    int lanes = 16;  // threads side by side on a run of positions: the head size rounded up to a power of two, 16 to 256
+    while (lanes < head_dim && lanes < 256) lanes *= 2;
+    const int threads = 256;
     if (dtype == FSIE_F32)
         pool_blocks_kernel<float><<<grid, threads, 0, stream>>>(
             static_cast<const float*>(k_pool), static_cast<const float*>(v_pool), block_tables, max_pages, page_size,
             static_cast<float*>(k_pooled), static_cast<float*>(v_pooled), pooled_tables, pooled_max_pages, pooled_page_size, jobs,
-            block_tokens, n_kv, head_dim);
+            block_tokens, n_kv, head_dim, lanes);
     else
         pool_blocks_kernel<bf16_t><<<grid, threads, 0, stream>>>(
             static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), block_tables, max_pages, page_size,
             static_cast<bf16_t*>(k_pooled), static_cast<bf16_t*>(v_pooled), pooled_tables, pooled_max_pages, pooled_page_size,
-            jobs, block_tokens, n_kv, head_dim);
+            jobs, block_tokens, n_kv, head_dim, lanes);
     FSIE_CHECK_LAUNCH("pool_blocks");
     return 0;
 }
