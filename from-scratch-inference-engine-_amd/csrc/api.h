@@ -74,7 +74,8 @@ int fsie_sandwich_norm(float* residual, const void* delta, const float* post_wei
 // out[t][h][:] = rmsnorm(o[t][h][:]; weight, eps) * act(gate[t][h][:]), a head `width` values wide; o float32, the sum
 // in order of n_planes arrays [n_tokens][heads * width] that lie one after the other
 int fsie_gated_headnorm(const float* o, int n_planes, const void* gate, int64_t gate_stride, const float* weight, void* out,
-                        int n_tokens, int heads, int width, float eps, int act, int dtype, hipStream_t stream);
+                        int n_tokens, int heads, int width, float eps, int act, int dtype, int64_t out_stride, float out_scale,
+                        hipStream_t stream);
 // x <- cap * tanh(x / cap) in place
 int fsie_softcap(float* x, int64_t n, float cap, hipStream_t stream);
 
@@ -154,7 +155,7 @@ int fsie_attention_prep(const void* proj, int64_t stride, int q_off, int k_off, 
                         int64_t pool_slots, int n_tokens, int dtype, int q_weight_stride, int v_unit_norm, float v_eps,
                         hipStream_t stream);
 int fsie_gate_heads(const void* x, int D, const float* gate, void* y, int n_tokens, int heads, int vdim, int dtype,
-                    hipStream_t stream);
+                    int64_t y_stride, float y_scale, hipStream_t stream);
 
 int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, int dtype,
               int out_f32, int kind, hipStream_t stream);

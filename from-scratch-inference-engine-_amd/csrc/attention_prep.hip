@@ -231,21 +231,24 @@ __global__ __launch_bounds__(kThreads) void attention_prep_values_kernel(
 // VEC: vdim and D are multiples of 4 and the arrays 16-byte aligned: a thread takes four values of a head
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void gate_heads_kernel(const T* __restrict__ x, int D, const float* __restrict__ gate,
-                                                              T* __restrict__ y, int heads, int vdim, int64_t total) {
+                                                              T* __restrict__ y, int heads, int vdim, int64_t total,
+                                                              int64_t y_stride, float y_scale) {
     constexpr int N = VEC ? 4 : 1;
     const int64_t e = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * N;
     if (e >= total) return;
     const int64_t th = e / vdim;  // token * heads + head
     const int j = static_cast<int>(e - th * vdim);
-    const float g = gate ? gate[th] : 1.f;
+    const float g = (gate ? gate[th] : 1.f) * y_scale;
+    const int64_t t = th / heads;
+    T* to = y + t * y_stride + (th - t * heads) * vdim + j;  // (rows of y may be columns of wider rows)
     if constexpr (VEC) {
         float a[4];
         load4(x + th * D + j, a);
 #pragma unroll
         for (int i = 0; i < 4; ++i) a[i] *= g;
-        store4(y + e, a);
+        store4(to, a);
     } else {
-        y[e] = from_float<T>(to_float(x[th * D + j]) * g);
+        *to = from_float<T>(to_float(x[th * D + j]) * g);
     }
 }
 
@@ -309,17 +312,20 @@ extern "C" int fsie_attention_prep(const void* proj, int64_t stride, int q_off, 
     return 0;
 }
 
-// y[t][h][0 .. vdim) = x[t][h][0 .. vdim) * gate[t][h] (gate null: 1), x's heads D values apart
+// y[t][h][0 .. vdim) = x[t][h][0 .. vdim) * gate[t][h] (gate null: 1) * y_scale, x's heads D values apart, y's rows y_stride
 extern "C" int fsie_gate_heads(const void* x, int D, const float* gate, void* y, int n_tokens, int heads, int vdim, int dtype,
-                               hipStream_t stream) {
-    FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && vdim > 0 && D >= vdim, "gate_heads: bad sizes");
+                               int64_t y_stride, float y_scale, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && vdim > 0 && D >= vdim && y_stride >= static_cast<int64_t>(heads) * vdim,
+                 "gate_heads: bad sizes");
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "gate_heads: unknown dtype %d", dtype);
     const int64_t total = static_cast<int64_t>(n_tokens) * heads * vdim;
     if (total == 0) return 0;
-    const bool vec = vdim % 4 == 0 && D % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const bool vec = vdim % 4 == 0 && D % 4 == 0 && y_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     const unsigned grid = static_cast<unsigned>(ceil_div64(vec ? total / 4 : total, kThreads));
 #define FSIE_GATE(T, V) \
-    gate_heads_kernel<T, V><<<grid, kThreads, 0, stream>>>(static_cast<const T*>(x), D, gate, static_cast<T*>(y), heads, vdim, total)
+    gate_heads_kernel<T, V><<<grid, kThreads, 0, stream>>>(static_cast<const T*>(x), D, gate, static_cast<T*>(y), heads, vdim, total, \
+                                                   y_stride, y_scale)
     if (dtype == FSIE_F32) {
         if (vec) FSIE_GATE(float, true); else FSIE_GATE(float, false);
     } else {

@@ -140,7 +140,8 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void gated_headnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
                                                                   int64_t gate_stride, const float* __restrict__ weight,
                                                                   T* __restrict__ out, int64_t n_runs, int heads, int width,
-                                                                  float eps, int act, int n_planes, int64_t plane) {
+                                                                  float eps, int act, int n_planes, int64_t plane,
+                                                                  int64_t out_stride, float out_scale) {
     const int lane = threadIdx.x & (FSIE_WAVE - 1);
     const int64_t run = static_cast<int64_t>(blockIdx.x) * (kThreads / FSIE_WAVE) + threadIdx.x / FSIE_WAVE;
     if (run >= n_runs) return;
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void gated_headnorm_kernel(const float* _
     const int h = static_cast<int>(run - t * heads);
     const float* src = o + (t * heads + h) * width;
     const T* g = gate + t * gate_stride + static_cast<int64_t>(h) * width;
-    T* dst = out + (t * heads + h) * width;
+    T* dst = out + t * out_stride + static_cast<int64_t>(h) * width;  // (rows of out may be columns of wider rows)
     // o comes as n_planes arrays a `plane` apart, added in order (the shares of a state kernel's row splits)
     auto value = [&](int i) {
         float x = src[i];
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(kThreads) void gated_headnorm_kernel(const float* _
     sum = wave_sum(sum);
     const float scale = 1.0f / sqrtf(sum / static_cast<float>(width) + eps);
     for (int i = lane; i < width; i += FSIE_WAVE)
-        dst[i] = from_float<T>(((value(i) * scale) * weight[i]) * gate_act(to_float(g[i]), act));
+        dst[i] = from_float<T>((((value(i) * scale) * weight[i]) * gate_act(to_float(g[i]), act)) * out_scale);
 }
 
 __global__ void softcap_kernel(float* __restrict__ x, int64_t n, float cap, float inv_cap) {
@@ -229,8 +230,9 @@ extern "C" int fsie_sandwich_norm(float* residual, const void* delta, const floa
 
 extern "C" int fsie_gated_headnorm(const float* o, int n_planes, const void* gate, int64_t gate_stride, const float* weight,
                                    void* out, int n_tokens, int heads, int width, float eps, int act, int dtype,
-                                   hipStream_t stream) {
+                                   int64_t out_stride, float out_scale, hipStream_t stream) {
     FSIE_REQUIRE(n_planes >= 1, "gated_headnorm: at least one plane of o");
+    FSIE_REQUIRE(out_stride >= static_cast<int64_t>(heads) * width, "gated_headnorm: rows of out shorter than the heads");
     const int64_t plane = static_cast<int64_t>(n_tokens) * heads * width;
     FSIE_REQUIRE(n_tokens >= 0 && heads > 0 && width > 0, "gated_headnorm: bad sizes T=%d heads=%d width=%d", n_tokens, heads,
                  width);
@@ -243,10 +245,12 @@ extern "C" int fsie_gated_headnorm(const float* o, int n_planes, const void* gat
     const unsigned grid = static_cast<unsigned>(ceil_div64(runs, kThreads / FSIE_WAVE));
     if (dtype == FSIE_F32) {
         gated_headnorm_kernel<float><<<grid, kThreads, 0, stream>>>(o, static_cast<const float*>(gate), gate_stride, weight,
-                                                                  static_cast<float*>(out), runs, heads, width, eps, act, n_planes, plane);
+                                                                  static_cast<float*>(out), runs, heads, width, eps, act, n_planes, plane,
+                                                                  out_stride, out_scale);
     } else {
         gated_headnorm_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(o, static_cast<const bf16_t*>(gate), gate_stride, weight,
-                                                                   static_cast<bf16_t*>(out), runs, heads, width, eps, act, n_planes, plane);
+                                                                   static_cast<bf16_t*>(out), runs, heads, width, eps, act, n_planes, plane,
+                                                                   out_stride, out_scale);
     }
     FSIE_CHECK_LAUNCH("gated_headnorm");
     return 0;

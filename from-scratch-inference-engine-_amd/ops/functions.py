@@ -824,12 +824,23 @@ def sandwich_norm(residual: torch.Tensor, delta: torch.Tensor, post_weight: torc
     return out
 
 
+def _columns_of(out: Optional[torch.Tensor], t: int, width: int, dtype, device, name: str) -> torch.Tensor:
+    """``out`` (or a new tensor) as the place of a result [t, width]: it may be a run of columns of wider rows."""
+    if out is None:
+        return torch.empty((t, width), dtype=dtype, device=device)
+    if (not out.is_cuda or out.dim() != 2 or tuple(out.shape) != (t, width) or out.dtype != dtype or out.stride(1) != 1
+            or out.stride(0) < width):
+        raise KernelError(f"{name} out: must be [{t}, {width}] of {dtype} on the GPU, rows contiguous (columns of wider rows may do)")
+    return out
+
+
 def gated_headnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int,
-                   act: str = "silu") -> torch.Tensor:
+                   act: str = "silu", out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
     """``rmsnorm(o[t, h]; weight, eps) * act(gate[t, h])`` for every token and head: ``o`` float32
     [T, heads * width] (or [P, T, heads * width]: planes that are added in order first), ``weight`` float32
     [width] (shared by the heads), ``gate`` [T, heads * width] in the activations' type (it may be columns of
-    wider rows); the result has the gate's type."""
+    wider rows); the result has the gate's type.  ``out``: where it goes (columns of wider rows may do); ``scale``: a
+    factor on it, applied before the one rounding."""
     if o.dim() == 2:
         o = o.unsqueeze(0)
     _need(o, "gated_headnorm o", dtype=torch.float32, ndim=3)
@@ -840,9 +851,10 @@ def gated_headnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, ep
         raise KernelError(f"gated_headnorm: rows of {total} values are not {heads} heads of {width}")
     if not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1 or tuple(gate.shape) != (t, total):
         raise KernelError("gated_headnorm gate: must be [T, heads * width] on the GPU with contiguous rows")
-    out = torch.empty((t, total), dtype=gate.dtype, device=o.device)
+    out = _columns_of(out, t, total, gate.dtype, o.device, "gated_headnorm")
     check(load().fsie_gated_headnorm(o.data_ptr(), planes, gate.data_ptr(), gate.stride(0), weight.data_ptr(), out.data_ptr(), t,
-                                     heads, width, float(eps), gate_act_code(act), dtype_code(gate.dtype), _stream()))
+                                     heads, width, float(eps), gate_act_code(act), dtype_code(gate.dtype), out.stride(0) if t else total,
+                                     float(scale), _stream()))
     return out
 
 
@@ -1109,17 +1121,19 @@ def attention_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off
     return q, gate
 
 
-def gate_heads(x: torch.Tensor, padded: int, vdim: int, heads: int, gate: Optional[torch.Tensor]) -> torch.Tensor:
+def gate_heads(x: torch.Tensor, padded: int, vdim: int, heads: int, gate: Optional[torch.Tensor],
+               out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
     """[T, heads * vdim]: of every head of ``x`` [T, heads * padded] its first ``vdim`` values times ``gate``
-    (float32 [T, heads]; None: as they are)."""
+    (float32 [T, heads]; None: as they are) times ``scale``.  ``out``: where it goes (columns of wider rows may do)."""
     _need(x, "gate_heads x", ndim=2)
     t = x.shape[0]
     if x.shape[1] != heads * padded or padded < vdim:
         raise KernelError(f"gate_heads: rows of {x.shape[1]} are not {heads} heads of {padded}")
     if gate is not None:
         _need(gate, "gate_heads gate", dtype=torch.float32, shape=(t, heads))
-    y = torch.empty((t, heads * vdim), dtype=x.dtype, device=x.device)
-    check(load().fsie_gate_heads(x.data_ptr(), padded, _ptr(gate), y.data_ptr(), t, heads, vdim, dtype_code(x.dtype), _stream()))
+    y = _columns_of(out, t, heads * vdim, x.dtype, x.device, "gate_heads")
+    check(load().fsie_gate_heads(x.data_ptr(), padded, _ptr(gate), y.data_ptr(), t, heads, vdim, dtype_code(x.dtype),
+                                 y.stride(0) if t else heads * vdim, float(scale), _stream()))
     return y
 
 

@@ -76,7 +76,7 @@ _SIGNATURES = {
     "fsie_gated_act": ([_P, _P, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_gemm_mfma_wide_gated": ([_P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_sandwich_norm": ([_P, _P, _P, c_float, _P, c_float, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
-    "fsie_gated_headnorm": ([_P, c_int, _P, c_int64, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int, _P], c_int),
+    "fsie_gated_headnorm": ([_P, c_int, _P, c_int64, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int, c_int64, c_float, _P], c_int),
     "fsie_gla_scan_shape": ([c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int),
                              ctypes.POINTER(c_int), ctypes.POINTER(c_int64)], c_int),
     "fsie_softcap": ([_P, c_int64, c_float, _P], c_int),
@@ -96,7 +96,7 @@ _SIGNATURES = {
     "fsie_attention_prep": ([_P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float,
                              c_int, _P, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, c_int, c_float,
                              _P], c_int),
-    "fsie_gate_heads": ([_P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_gate_heads": ([_P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int64, c_float, _P], c_int),
     "fsie_group_rmsnorm": ([_P, _P, c_int, _P, c_int, c_float, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, c_int, c_int,
                             _P], c_int),
     "fsie_causal_conv": ([_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],

@@ -775,7 +775,19 @@ class GQAttention(Mixer):
             ops.rope_kv_write(qkv, ctx.positions, nh, nkv, hd, None, bias=bias, **store)  # (no rotation: bias, write)
         return qkv
 
-    def _forward_prepared(self, x: torch.Tensor, ctx, cache, plan) -> torch.Tensor:
+    @property
+    def heads_width(self) -> int:
+        """Values a token has behind attention, in front of the output projection."""
+        return self.n_heads * self.value_dim
+
+    def forward_heads(self, x: torch.Tensor, ctx, cache, out: torch.Tensor, scale: float = 1.0) -> None:
+        """``forward`` without the output projection: the heads' results times ``scale`` into ``out`` [T, heads_width]
+        (columns of wider rows may do).  For a mixer that runs this one beside another and projects both at once."""
+        if not self.prepared:
+            raise NotImplementedError("attention: the heads' results alone come from the one-kernel path (fused_prep=True)")
+        self._forward_prepared(x, ctx, cache, ctx.plan(self.planner()), heads_out=out, heads_scale=scale)
+
+    def _forward_prepared(self, x: torch.Tensor, ctx, cache, plan, heads_out=None, heads_scale: float = 1.0):
         """Gate, mixed values or values of another size than the keys: the fused projection, one kernel for all
         that stands between it and attention, attention over heads of ``padded`` values, the gate."""
         nh, nkv, hd, vd, pd = self.n_heads, self.n_kv, self.head_dim, self.value_dim, self.padded
@@ -815,6 +827,9 @@ class GQAttention(Mixer):
             pooled = (blocks.k_pool, blocks.v_pool, blocks.block_tables, self.pool)
         out = paged_attention(q, nh * pd, cache, plan, nh, nkv, pd, self.window, self.scale, x.shape[0], sinks=self.sink,
                               share_keys=self.share_keys, softcap=self.softcap, pooled=pooled)
+        if heads_out is not None:
+            ops.gate_heads(out, pd, vd, nh, gate, out=heads_out, scale=heads_scale)
+            return None
         if gate is not None or pd != vd:
             out = ops.gate_heads(out, pd, vd, nh, gate)
         return self.o.for_residual(out, ctx)

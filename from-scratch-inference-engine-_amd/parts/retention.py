@@ -72,26 +72,59 @@ class Retention(Mixer):
     def cache_need(self) -> StateNeed:
         return StateNeed((self.n_heads, self.key_dim, self.value_dim), "float32")
 
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+    @property
+    def heads_width(self) -> int:
+        """Values a token has behind the gate, in front of the output projection."""
+        return self.v_width
+
+    def forward_heads(self, x: torch.Tensor, ctx, cache, out: torch.Tensor, scale: float = 1.0) -> None:
+        """``forward`` without the output projection: the gated heads times ``scale`` into ``out`` [T, heads_width]
+        (columns of wider rows may do)."""
+        self.forward(x, ctx, cache, heads_out=out, heads_scale=scale)
+
+    def forward(self, x: torch.Tensor, ctx, cache, heads_out=None, heads_scale: float = 1.0):
         kw, vw = self.k_width, self.v_width
         p = self.qkvg(x)
         # (the scan's own first kernel turns q and k by the step's cosines and sines as it reads them)
         table = self.position.table(ctx) if self.position.rotates else None
         o = ops.gla_scan(p, 0, kw, 2 * kw, None, cache.state, ctx.q_starts, ctx.seq_slots, self.n_heads, self.key_dim,
                          self.value_dim, self.key_scale, 1.0, head_decay=self._decay, cos_sin=table)
-        y = ops.gated_headnorm(o, p[:, 2 * kw + vw:], self._ones, self.norm_eps, self.n_heads, self.gate_activation)
-        return self.o.for_residual(y, ctx)
+        y = ops.gated_headnorm(o, p[:, 2 * kw + vw:], self._ones, self.norm_eps, self.n_heads, self.gate_activation,
+                               out=heads_out, scale=heads_scale)
+        return None if heads_out is not None else self.o.for_residual(y, ctx)
 
 
 @register_part("mixer", "side_by_side")
 class SideBySide(Mixer):
     """Two mixers that read the same input; the result is left_scale * left(x) + right_scale * right(x), summed in
     float32.  What the two keep for a request are two caches: ``cache_need`` names them ``left`` and ``right`` and
-    ``forward`` gets the views under the same names."""
+    ``forward`` gets the views under the same names.
 
-    def __init__(self, left: Mixer, right: Mixer, left_scale: float = 1.0, right_scale: float = 1.0):
+    Where both mixers end in an output projection without bias and can hand over what stands in front of it
+    (``forward_heads``, ``heads_width``, a ``Linear`` named ``o``), the two projections are one: the mixers write their
+    heads, times their scales, side by side into one row a token, and one product with [W_o left | W_o right] gives the
+    sum (the scales multiply the activations in float32, before their one rounding).  ``joint_output=False`` keeps two
+    products and a kernel for the weighted sum."""
+
+    def __init__(self, left: Mixer, right: Mixer, left_scale: float = 1.0, right_scale: float = 1.0, joint_output: bool = True):
         self.left, self.right = left, right
         self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+
+        def joins(m) -> bool:
+            return (callable(getattr(m, "forward_heads", None)) and isinstance(getattr(m, "o", None), Linear) and not m.o.has_bias
+                    and getattr(m, "prepared", True))
+        self.joint = bool(joint_output) and joins(left) and joins(right) and left.o.out_features == right.o.out_features
+        self.o = Linear(left.heads_width + right.heads_width, left.o.out_features) if self.joint else None
+
+    def prepare(self, device, compute_dtype) -> None:
+        if self.joint and self.o.weight is None:
+            # (the mixers' own prepare runs after this one: they find their projections' weights gone and make no copies)
+            self.o.weight = torch.cat([self.left.o.weight, self.right.o.weight], dim=1).contiguous()
+            self.left.o.weight = self.right.o.weight = None
+            self.o.prepare(bool(self.options.get("weight_copies", True)))
+
+    def release_optional_memory(self) -> int:
+        return self.o.drop_copy() if self.joint else 0
 
     @property
     def graph_safe(self) -> bool:
@@ -113,6 +146,12 @@ class SideBySide(Mixer):
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         cache = cache or {}
+        if self.joint:
+            wl = self.left.heads_width
+            heads = torch.empty((x.shape[0], self.o.in_features), dtype=x.dtype, device=x.device)
+            self.left.forward_heads(x, ctx, cache.get("left"), heads[:, :wl], self.left_scale)
+            self.right.forward_heads(x, ctx, cache.get("right"), heads[:, wl:], self.right_scale)
+            return self.o.for_residual(heads, ctx)
         whole = ctx.partial_sums_ok
         ctx.partial_sums_ok = False  # (both results are added here: each comes whole, not as partial sums)
         try:

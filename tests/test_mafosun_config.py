@@ -37,7 +37,7 @@ def test_what_the_builder_makes():
     blocks = spec.layers
     assert [type(b).__name__ for b in blocks] == ["BranchNormBlock"] * 4 and blocks[2].ffn is None
     pair = blocks[0].mixer
-    assert pair.left_scale == 1.3 and pair.right_scale == 0.4
+    assert pair.left_scale == 1.3 and pair.right_scale == 0.4 and pair.joint and pair.o.in_features == 6 * 40 + 3 * 16
     assert pair.cache_need() == {"left": PagedNeed(3, 48, 16, 0), "right": StateNeed((3, 24, 16), "float32")}
     assert pair.left.chunk == 16 and pair.left.value_unit_norm_eps == 1e-6 and not pair.left.position.rotates
     assert pair.right.decay == [0.9, 0.99, 1.0] and pair.right.position.rotary_dim == 16

@@ -499,11 +499,12 @@ CONFIG_A = {"architecture": "Mafosun", "width": 72, "vocab": 150, "norm": {"eps"
     layer("attention", attention(2, 1, 16, 16, 0.3, 5, 7, None, rotation(77.0, 16)), None),
     layer("parallel", side_by_side(attention(2, 2, 16, 16, 0.4, 33), retention_of(2, 40, 36, (0.5, 0.999)), 1.0, 1.0), dense(50)),
 ]}
-# B: attention only; no rotation in one layer, one kv head a query head, blocks and a window of one position, top 1,
-#    one group
+# B: attention only; no rotation in one layer, one kv head a query head, blocks and a window of one position, a window
+#    without blocks, top 1, one group
 CONFIG_B = {"architecture": "Mafosun", "width": 64, "vocab": 97, "norm": {"eps": 1e-5}, "layers": [
     layer("attention", attention(4, 4, 16, 24, 0.3, 1, 1, 3.0), moe(24, 1, 1, 1, 1)),
     layer("attention", attention(4, 1, 32, 32, 0.2, 12, 12, 30.0, rotation(10000.0, 32, (8.0, 1.0, 4.0, 32))), moe(32, 5, 1, 1, 1)),
+    layer("attention", attention(2, 2, 48, 48, 0.15, 21, None, None, rotation(200.0, 24)), dense(72)),  # a window alone
 ]}
 # C: two mixers side by side only, heads of sizes the matrix-core kernels take, a chunk of one page, every head with
 #    its own decay, all experts chosen
@@ -731,6 +732,37 @@ def test_model_whole_in_portions_decoded_and_batched(models, name, dtype):
     for r in seqs:
         check(got, r, f"{name} batched {r}")
     assert all(a.pages_issued_again() for a in runner.manager.allocators)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_output_product_or_two_for_mixers_side_by_side(models, dtype):
+    """The mixers of a side-by-side layer share one output product over their heads laid side by side, the scales on the
+    activations; with ``joint_output`` off they keep their own products and a kernel adds the results.  Both are the
+    plain model's logits."""
+    from pathlib import Path
+
+    from from_scratch_inference_engine_amd.config.base import read_config_json
+    from from_scratch_inference_engine_amd.engine.model import Model, Runner
+    from from_scratch_inference_engine_amd.models.registry import build_model_spec, parse_config
+    from from_scratch_inference_engine_amd.parts import SideBySide
+    from from_scratch_inference_engine_amd.weights.loader import load_weights
+
+    d, cfg, w = models["C" if dtype == "float32" else "C~"]
+    ids = helpers.token_ids(cfg["vocab"], 45, 9)
+    ref = plain.forward(cfg, w, ids)
+    for joint in (True, False):
+        spec = build_model_spec(parse_config(read_config_json(d)))
+        pairs = [b.mixer for b in spec.layers if isinstance(b.mixer, SideBySide)]
+        assert pairs and all(m.joint for m in pairs)
+        if not joint:
+            for m in pairs:
+                m.joint, m.o = False, None
+        model = Model(spec, dtype, "cuda:0")
+        load_weights(Path(d), spec.bindings, model.dtype, model.device, spec.ignore_unexpected)
+        model._prepare(True)
+        runner = Runner(model, page_size=8, num_pages=40, max_requests=2)
+        got = step_through(runner, [[("a", 30)], [("a", 2)]] + [[("a", 1)]] * 13, {"a": ids})["a"]
+        close_enough(got, ref, dtype, f"joint {joint}")
 
 
 def test_long_decoding_with_a_far_first_token(models):
