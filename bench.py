@@ -290,14 +290,14 @@ def mafosun_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
     two groups (two a token, from the best group) in turn; an expert has gate, up and down of ff / 8, so a token's two
     experts are a quarter of the dense feed-forward's arithmetic."""
     heads = width // 128
-    bands = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
-    gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
+    bands = {"factor": 4.0, "low": 1.0, "high": 8.0, "original": 4096}
+    gqa = {"heads": heads, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
            "mask": {"size": 1024, "pool": 64}, "rot": {"base": 500000.0, "dims": 64, "scaling": bands}}
     pair = {"left": {"heads": heads // 2, "kv_heads": max(1, width // 1024), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
                      "mask": {"size": 1024}},
             "right": {"heads": width // 256, "dim": 128, "vdim": 128, "rot": {"base": 500000.0, "dims": 128},
-                      "decay": [1.0 - 2.0 ** -(5 + i % 6) for i in range(width // 256)]},
-            "left_scale": 1.2, "right_scale": 0.5}
+                      "decay": [1.0 - 2.0 ** -(4 + i % 5) for i in range(width // 256)]},
+            "left_scale": 0.8, "right_scale": 0.7}
     dense = {"kind": "dense", "ff": ff}
     routed = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 8, "top": 2, "groups": {"count": 2, "keep": 1}}}
     out = [{"type": "parallel" if i % 2 == 0 else "attention", "mixer": dict(pair if i % 2 == 0 else gqa),

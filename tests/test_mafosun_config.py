@@ -75,7 +75,7 @@ def test_refusals(edit, word):
 
 
 def test_rescaled_frequencies():
-    for dims, base, bands in ((64, 250000.0, (8.0, 1.0, 4.0, 1024)), (20, 1000.0, (4.0, 1.0, 4.0, 64)), (6, 50.0, (2.0, 0.5, 3.0, 16))):
+    for dims, base, bands in ((64, 300000.0, (6.0, 1.0, 3.0, 2048)), (20, 1000.0, (4.0, 1.0, 4.0, 64)), (6, 50.0, (2.0, 0.5, 3.0, 16))):
         enc = RotaryEncoding(dims + 4, base, rotary_dim=dims, bands=bands)
         ref = plain.rotary_frequencies(dims, base, dict(zip(("factor", "low", "high", "original"), bands)))
         assert np.allclose(enc.frequencies(), ref, rtol=1e-14, atol=0)
@@ -92,7 +92,7 @@ def visible_by_definition(pos, window, chunk, pool):
 
 
 @pytest.mark.parametrize("window, chunk, pool", [(None, 16, None), (None, 1, None), (None, 7, None), (10, None, 4), (5, None, 7), (1, None, 1),
-                                                 (96, None, 12), (None, None, None)])
+                                                 (80, None, 10), (None, None, None)])
 @pytest.mark.parametrize("units", [1, 256])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_plan_covers_what_a_query_reads(window, chunk, pool, units, dtype):
