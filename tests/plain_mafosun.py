@@ -89,7 +89,7 @@ def rotate(x, positions, freqs, dims, layout):
     (i, i + dims/2) ('half')."""
     out = x.copy()
     ang = positions[:, None].astype(np.float64) * freqs[None, :]  # [T, dims/2]
-    c, s = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+    c, s = np.cos(ang)[:, None, :].astype(x.dtype), np.sin(ang)[:, None, :].astype(x.dtype)  # (the inputs' type: float64 here)
     if layout == "interleaved":
         a, b = x[..., 0:dims:2], x[..., 1:dims:2]
         out[..., 0:dims:2] = a * c - b * s
@@ -108,7 +108,7 @@ def window_pool_attention(q, k, v, scale, window, pool, softcap, sink):
     to the softmax's denominator."""
     t, heads, _ = q.shape
     group = heads // k.shape[1]
-    out = np.zeros((t, heads, v.shape[2]))
+    out = np.zeros((t, heads, v.shape[2]), dtype=v.dtype)
     n_blocks = t // pool if pool else 0
     if n_blocks:
         kp = k[:n_blocks * pool].reshape(n_blocks, pool, *k.shape[1:]).mean(1)
@@ -135,7 +135,7 @@ def chunk_attention(q, k, v, scale, chunk):
     """Query i sees keys j <= i of its own chunk (floor(i / chunk) == floor(j / chunk)); ordinary softmax."""
     t, heads, _ = q.shape
     group = heads // k.shape[1]
-    out = np.zeros((t, heads, v.shape[2]))
+    out = np.zeros((t, heads, v.shape[2]), dtype=v.dtype)
     for i in range(t):
         lo = i // chunk * chunk
         for h in range(heads):
@@ -149,9 +149,9 @@ def chunk_attention(q, k, v, scale, chunk):
 def retention(q, k, v, decay):
     """S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, per head; q, k [T, H, d], v [T, H, e]."""
     t, heads, d = q.shape
-    out = np.zeros((t, heads, v.shape[2]))
+    out = np.zeros((t, heads, v.shape[2]), dtype=v.dtype)
     for h in range(heads):
-        state = np.zeros((d, v.shape[2]))
+        state = np.zeros((d, v.shape[2]), dtype=v.dtype)
         for i in range(t):
             state = decay[h] * state + np.outer(k[i, h], v[i, h])
             out[i, h] = state.T @ q[i, h]
